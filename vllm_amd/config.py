@@ -111,6 +111,28 @@ class ModelSpec:
     # BART-style TEXT encoder-decoder (architecture "bart"): layers of
     # the bidirectional text encoder; decoder fields above.
     encoder_layers: int = 0
+    # Heterogeneous layer stacks (architecture "gadilix"): one dict per
+    # layer — {"type", "mixer": {...}, "mlp": {...} | None, and
+    # optionally "weights_of": j} — read verbatim from config.json.
+    # None for the homogeneous families above, whose flat fields
+    # describe every layer.
+    layer_specs: Optional[list] = None
+    # Multiplier on every sublayer's contribution to the residual sum.
+    residual_mult: float = 1.0
+
+    @property
+    def has_token_shift(self) -> bool:
+        """Every layer keeps the previous token's mixer input as
+        per-request state (one row per running request and layer)."""
+        return self.architecture == "gadilix"
+
+    @property
+    def has_row_state(self) -> bool:
+        """Per-request state that lives in runner rows rather than in
+        paged blocks (SSM state, token-shift carry). Such state is not
+        content-addressable, so prefix caching is off for these models
+        and rows are cleared on (re)admission."""
+        return self.has_mamba or self.has_token_shift
 
     @property
     def is_moe(self) -> bool:
@@ -1011,11 +1033,58 @@ MODEL_PRESETS: dict[str, ModelSpec] = {
 }
 
 
+def _gadilix_spec(path: str, cfg: dict) -> ModelSpec:
+    """Gadilix config.json: {"architecture", "vocab", "width",
+    "residual_mult", "norm": {"eps"}, "layers": [...]}. Every size and
+    constant is per layer; the flat attention fields mirror the widest
+    layer only so that generic sizing code has something sane to read."""
+    layers = cfg["layers"]
+    if not layers:
+        raise ValueError("gadilix: config lists no layers")
+    for i, entry in enumerate(layers):
+        if entry.get("type") != "attention":
+            raise ValueError(
+                f"gadilix: layer {i} has unknown mixer type "
+                f"{entry.get('type')!r}")
+        j = entry.get("weights_of")
+        if j is not None and (not 0 <= j < len(layers)
+                              or layers[j].get("weights_of") is not None):
+            raise ValueError(
+                f"gadilix: layer {i} borrows weights of layer {j}, which "
+                "is not a layer with tensors of its own")
+        mlp = entry.get("mlp")
+        if mlp is not None and mlp.get("kind") != "moe":
+            raise ValueError(
+                f"gadilix: layer {i} has unknown mlp kind "
+                f"{mlp.get('kind')!r}")
+    mixers = [e["mixer"] for e in layers]
+    return ModelSpec(
+        name=os.path.basename(path.rstrip("/")) or "gadilix",
+        architecture="gadilix",
+        vocab_size=cfg["vocab"],
+        hidden_size=cfg["width"],
+        intermediate_size=0,
+        num_layers=len(layers),
+        num_heads=max(m["heads"] for m in mixers),
+        num_kv_heads=max(m["kv_heads"] for m in mixers),
+        head_dim=max(max(m["dim"], m["vdim"]) for m in mixers),
+        rms_norm_eps=cfg["norm"]["eps"],
+        # Positions never enter the computation: no table bounds them.
+        max_position_embeddings=1 << 24,
+        layer_specs=layers,
+        residual_mult=float(cfg.get("residual_mult", 1.0)),
+        eos_token_id=-1,
+        bos_token_id=0,
+    )
+
+
 def _spec_from_hf_config(path: str) -> ModelSpec:
     """Build a ModelSpec from a local HF config.json directory/file."""
     cfg_path = path if path.endswith(".json") else os.path.join(path, "config.json")
     with open(cfg_path) as f:
         hf = json.load(f)
+    if str(hf.get("architecture", "")).lower() == "gadilix":
+        return _gadilix_spec(path, hf)
     arch = (hf.get("architectures") or ["LlamaForCausalLM"])[0].lower()
     if "jamba" in arch:
         # HF JambaForCausalLM: hybrid attn/mamba layer pattern + SSM

@@ -26,6 +26,8 @@ class NewRequestData:
     # Window-group block ids (mixed sliding+global models); None for
     # single-group models.
     block_ids_w: object = None
+    # Streamed prompt still open: reaching its end samples nothing.
+    prompt_open: bool = False
 
 
 @dataclass(slots=True)
@@ -42,6 +44,9 @@ class CachedRequestData:
     # Parallel to new_block_ids for the window group (mixed models);
     # entries are None for single-group models.
     new_block_ids_w: list = field(default_factory=list)
+    # Parallel to req_ids when any request streams its prompt (else
+    # empty): whether the prompt is still open after this step's tokens.
+    prompt_open: list[bool] = field(default_factory=list)
 
     @property
     def num_reqs(self) -> int:
@@ -65,6 +70,9 @@ class SchedulerOutput:
     # prefix block; ("in", gpu_block_id, host_slot) = H2D restore of a
     # host-tier prefix hit.
     kv_swap_ops: list[tuple[str, int, int]] = field(default_factory=list)
+    # req_id -> offsets into this step's tokens of that request whose
+    # raw logits go back to the client (ModelRunnerOutput.tapped_logits).
+    logit_taps: dict[str, list[int]] = field(default_factory=dict)
 
     @property
     def num_reqs(self) -> int:
@@ -91,6 +99,9 @@ class ModelRunnerOutput:
     # Prompt logprobs computed this step (chunked-prefill order):
     # req_id -> one {token_id: logprob} dict per prompt position covered.
     prompt_logprobs: Optional[dict[str, list[dict[int, float]]]] = None
+    # Raw logits at the tapped positions: req_id -> fp32 CPU tensor
+    # [taps, vocab], rows in the order of SchedulerOutput.logit_taps.
+    tapped_logits: Optional[dict] = None
 
 
 EMPTY_MODEL_RUNNER_OUTPUT = ModelRunnerOutput(req_ids=[], sampled_token_ids=[])
@@ -106,6 +117,7 @@ class EngineCoreOutput:
     new_logprobs: Optional[list[dict[int, float]]] = None
     new_prompt_logprobs: Optional[list[dict[int, float]]] = None
     pooled: Optional[list[float]] = None
+    tapped_logits: object = None  # fp32 CPU tensor [taps, vocab]
 
     @property
     def finished(self) -> bool:

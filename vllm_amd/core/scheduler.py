@@ -129,7 +129,7 @@ class Scheduler:
                           if spec.sliding_window > 0
                           and spec.global_attn_every_n_layers == 0 else 0)
         enable_caching = config.cache_config.enable_prefix_caching
-        if spec.has_mamba or spec.pooling_only:
+        if spec.has_row_state or spec.pooling_only:
             # Defense in depth (EngineArgs also clears the flag): SSM
             # state is not content-addressable and encoders need every
             # position's hidden state — a prefix hit would skip tokens
@@ -173,6 +173,21 @@ class Scheduler:
         self.requests[request.request_id] = request
         request.status = RequestStatus.WAITING
         self.waiting.append(request)
+
+    def extend_prompt(self, req_id: str, token_ids: list[int],
+                      logit_taps: Optional[list[int]] = None,
+                      close: bool = False) -> None:
+        """Append prompt tokens to a request admitted with
+        prompt_open=True (streamed input). logit_taps are absolute
+        positions; close=True ends the stream, after which the request
+        samples like any other once its prompt is computed."""
+        request = self.requests[req_id]
+        request.extend_prompt(token_ids)
+        if logit_taps:
+            request.logit_taps = sorted(set(request.logit_taps)
+                                        | set(logit_taps))
+        if close:
+            request.prompt_open = False
 
     def finish_requests(
         self, request_ids: list[str], status: RequestStatus
@@ -235,6 +250,7 @@ class Scheduler:
         # Precondition scan (no mutation).
         for r in running:
             if (r.spec_token_ids or r.grammar is not None
+                    or r.prompt_open or r.logit_taps
                     or r.num_tokens + r.num_output_placeholders
                     - r.num_computed_tokens != 1
                     or r.num_computed_tokens + 1 > max_len):
@@ -305,6 +321,7 @@ class Scheduler:
         cached = CachedRequestData()
         num_scheduled_tokens: dict[str, int] = {}
         preempted_reqs: set[str] = set()
+        logit_taps: dict[str, list[int]] = {}
 
         # ---- RUNNING loop (reference scheduler.py:484) ----
         req_index = 0
@@ -358,6 +375,11 @@ class Scheduler:
                 self.kv_cache_manager.last_w_block_ids(
                     request.request_id, len(new_blocks)))
             cached.num_computed_tokens.append(request.num_computed_tokens)
+            taps = request.take_logit_taps(
+                request.num_computed_tokens,
+                request.num_computed_tokens + num_new_tokens)
+            if taps:
+                logit_taps[request.request_id] = taps
             # Tokens the runner hasn't seen yet: any output tokens generated
             # since the prompt (runner keeps its own copy; for non-resumed
             # requests only the newest token is unseen).
@@ -377,7 +399,8 @@ class Scheduler:
             # the next schedule() may run before this step's results).
             request.num_computed_tokens += num_new_tokens
             if (request.num_computed_tokens
-                    == request.num_tokens + request.num_output_placeholders):
+                    == request.num_tokens + request.num_output_placeholders
+                    and not request.prompt_open):
                 request.num_output_placeholders += 1
             req_index += 1
 
@@ -456,6 +479,10 @@ class Scheduler:
             all_block_ids_w = self.kv_cache_manager.get_block_ids_w(
                 request.request_id
             )
+            taps = request.take_logit_taps(
+                num_computed, num_computed + num_new_tokens)
+            if taps:
+                logit_taps[request.request_id] = taps
             if resumed:
                 cached.req_ids.append(request.request_id)
                 cached.resumed.append(True)
@@ -475,15 +502,20 @@ class Scheduler:
                         lora_id=request.lora_id,
                         mm_data=request.mm_data,
                         block_ids_w=all_block_ids_w,
+                        prompt_open=request.prompt_open,
                     )
                 )
             num_scheduled_tokens[request.request_id] = num_new_tokens
             token_budget -= num_new_tokens
             request.num_computed_tokens += num_new_tokens
             if (request.num_computed_tokens
-                    == request.num_tokens + request.num_output_placeholders):
+                    == request.num_tokens + request.num_output_placeholders
+                    and not request.prompt_open):
                 request.num_output_placeholders += 1
 
+        if any(self.requests[r].prompt_open for r in cached.req_ids):
+            cached.prompt_open = [self.requests[r].prompt_open
+                                  for r in cached.req_ids]
         total = sum(num_scheduled_tokens.values())
         out = SchedulerOutput(
             scheduled_new_reqs=scheduled_new_reqs,
@@ -493,6 +525,7 @@ class Scheduler:
             finished_req_ids=self.finished_req_ids,
             scheduled_spec_decode_tokens=scheduled_spec_tokens,
             kv_swap_ops=self.kv_cache_manager.take_swap_ops(),
+            logit_taps=logit_taps,
         )
         self.finished_req_ids = set()
         return out
@@ -552,6 +585,13 @@ class Scheduler:
                     request.prompt_logprob_chunks = (
                         getattr(request, "prompt_logprob_chunks", [])
                         + new_plp)
+
+            if runner_output.tapped_logits:
+                tapped = runner_output.tapped_logits.get(req_id)
+                if tapped is not None:
+                    outputs.append(EngineCoreOutput(
+                        req_id=req_id, new_token_ids=[],
+                        tapped_logits=tapped))
 
             new_token_ids = sampled_by_req.get(req_id) or []
             num_spec_sched = (len(spec_sched.get(req_id, ()))

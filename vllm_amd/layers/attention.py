@@ -98,3 +98,69 @@ class Attention(nn.Module):
             )
             out[s:e] = o.transpose(0, 1).to(out.dtype)
         return out
+
+
+class PooledWindowAttention(nn.Module):
+    """Sliding-window attention whose far context is kept as pooled
+    blocks: position i attends the `window` most recent tokens and, for
+    every block of `pool` consecutive tokens that lies wholly before
+    that window, ONE key/value — the block's mean key and mean value.
+    Window tokens and pooled blocks share one softmax. Positions do not
+    enter the scores. Key and value head widths may differ.
+
+    Cache per layer (allocated by the runner, paged by the same block
+    table as every other model): k [blocks, G, block_size, D],
+    v [blocks, G, block_size, Dv], and fp32 pooled areas
+    [blocks, G, ceil(block_size / pool), D|Dv]; a pooled block is stored
+    with the page that holds its last position, so it lives and dies
+    with that page. Each step writes the new K/V, finalizes the pooled
+    blocks the step completed (means of the keys as cached), then runs
+    the varlen attention op over decodes and prefill chunks together.
+
+    An optional per-head output gate (logits [T, H]) is applied in the
+    attention epilogue: out[t, h] *= sigmoid(gate[t, h])."""
+
+    def __init__(self, num_heads: int, head_dim: int, v_head_dim: int,
+                 scale: float, num_kv_heads: int, window: int, pool: int):
+        super().__init__()
+        assert num_heads % num_kv_heads == 0
+        assert window >= 1 and pool >= 1
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.v_head_dim = v_head_dim
+        self.scale = scale
+        self.window = window
+        self.pool = pool
+
+    def forward(self, q, k, v, gate, cache_idx: int) -> torch.Tensor:
+        """q [T, H, D], k [T, G, D], v [T, G, Dv], gate [T, H] or None
+        (all may be strided slices of one fused projection) ->
+        [T, H * Dv]."""
+        ctx = get_forward_context()
+        meta = ctx.attn_metadata
+        T = q.shape[0]
+        if not ctx.kv_caches:
+            return self._profile_attention(q, k, v, gate, meta)
+        k_cache, v_cache, pool_k, pool_v = ctx.kv_caches[cache_idx]
+        ops.split_cache_write(k, v, k_cache, v_cache, meta.slot_mapping)
+        ops.pool_update(k_cache, v_cache, pool_k, pool_v, meta.block_table,
+                        meta.query_start_loc, meta.seq_lens, self.pool,
+                        max_query_len=meta.max_query_len)
+        out = ops.pooled_window_attention(
+            q, k_cache, v_cache, pool_k, pool_v, meta.block_table,
+            meta.query_start_loc, meta.seq_lens, self.scale, self.window,
+            self.pool, gate=gate, num_decodes=meta.num_decodes,
+            max_seq_len=meta.max_seq_len,
+            max_query_len=meta.max_query_len)
+        return out.reshape(T, -1)
+
+    def _profile_attention(self, q, k, v, gate, meta) -> torch.Tensor:
+        """Memory-profiling run (no cache): only the activation footprint
+        matters, so attend each token to itself."""
+        group = self.num_heads // self.num_kv_heads
+        out = v.repeat_interleave(group, dim=1)
+        if gate is not None:
+            out = out * torch.sigmoid(gate.float()).unsqueeze(-1).to(
+                out.dtype)
+        return out.reshape(q.shape[0], -1)

@@ -39,6 +39,7 @@ class FusedMoE(nn.Module):
         dtype: torch.dtype = None,
         enable_expert_parallel: bool = False,
         eplb_window: int = 0,
+        learned_router: bool = True,
     ):
         super().__init__()
         from vllm_amd.parallel.state import get_ep_group
@@ -67,8 +68,11 @@ class FusedMoE(nn.Module):
         self.top_k = top_k
         self.renormalize = renormalize
         self.activation = activation
-        self.gate = ReplicatedLinear(hidden_size, num_experts, bias=False,
-                                     dtype=dtype)
+        # learned_router=False: the caller routes (e.g. a
+        # TokenTableRouter) and calls run_experts() directly.
+        self.gate = (ReplicatedLinear(hidden_size, num_experts, bias=False,
+                                      dtype=dtype)
+                     if learned_router else None)
         # TP: [E, 2*I/tp, H]; EP: [E/ep, 2*I, H].
         self.w13 = nn.Parameter(
             torch.empty(self.num_local_experts, 2 * self.i_shard,
@@ -300,3 +304,22 @@ class FusedMoE(nn.Module):
         self.w13.data[:, :i] = w1_full[:, r * i:(r + 1) * i]
         self.w13.data[:, i:] = w3_full[:, r * i:(r + 1) * i]
         self.w2.data.copy_(w2_full[:, :, r * i:(r + 1) * i])
+
+
+class TokenTableRouter(nn.Module):
+    """Routing without a learned gate: a fixed integer table
+    [vocab, top_k] names each token id's experts (distinct per row);
+    every chosen expert gets weight 1/top_k. Output feeds
+    FusedMoE.run_experts like any other router's (weights, ids)."""
+
+    def __init__(self, vocab_size: int, top_k: int):
+        super().__init__()
+        self.top_k = top_k
+        self.register_buffer(
+            "table", torch.zeros(vocab_size, top_k, dtype=torch.int32))
+
+    def forward(self, input_ids: torch.Tensor):
+        ids = self.table[input_ids]
+        weights = torch.full(ids.shape, 1.0 / self.top_k,
+                             dtype=torch.float32, device=ids.device)
+        return weights, ids

@@ -49,3 +49,27 @@ class LayerNorm(nn.Module):
         if residual is not None:
             return out, residual
         return out
+
+
+class ScalarRMSNorm(nn.Module):
+    """RMS norm whose gain is ONE number for all coordinates:
+    x / sqrt(mean(x^2) + eps) * g. Always computed in fp32.
+
+    forward(x) returns the normed rows (fp32, or out_dtype);
+    add_into(residual, y, mult) does residual += mult * norm(y) in place
+    on an fp32 residual stream and can hand back a copy of the updated
+    residual in the compute dtype for the next GEMM (one fused pass)."""
+
+    def __init__(self, eps: float = 1e-6):
+        super().__init__()
+        self.gain = nn.Parameter(torch.ones((), dtype=torch.float32),
+                                 requires_grad=False)
+        self.eps = eps
+
+    def forward(self, x: torch.Tensor, out_dtype=None) -> torch.Tensor:
+        return ops.scalar_rms_norm(x, self.gain, self.eps, out_dtype)
+
+    def add_into(self, residual: torch.Tensor, y: torch.Tensor,
+                 mult: float, out_dtype=None) -> torch.Tensor:
+        return ops.add_scaled_scalar_norm(residual, y, self.gain,
+                                          self.eps, mult, out_dtype)

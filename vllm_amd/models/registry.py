@@ -49,6 +49,10 @@ def get_model_class(architecture: str):
         from vllm_amd.models.mamba import MambaForCausalLM
 
         return MambaForCausalLM
+    if architecture == "gadilix":
+        from vllm_amd.models.gadilix import GadilixForCausalLM
+
+        return GadilixForCausalLM
     if architecture == "deepseek":
         from vllm_amd.models.deepseek import DeepseekForCausalLM
 
@@ -112,6 +116,11 @@ def initialize_dummy_weights(model: torch.nn.Module, seed: int = 0) -> None:
             continue
         val = gen_full(name, tuple(param.shape))
         param.data.copy_(val.to(param.dtype))
+    # Families with state the generic rules cannot fill (integer
+    # routing tables, scalar gains) finish their own dummy init.
+    finish = getattr(model, "finish_dummy_init", None)
+    if finish is not None:
+        finish(seed)
 
 
 def load_model(config: ModelConfig, device: torch.device) -> torch.nn.Module:

@@ -169,3 +169,51 @@ def fused_moe(hidden, w13, w2, topk_weights, topk_ids, activation="silu",
     return backend.fused_moe(hidden, w13, w2, topk_weights, topk_ids,
                              activation, w13_shuf=w13_shuf,
                              w2_shuf=w2_shuf)
+
+
+# ---------------------------------------------------------------------
+# fp32 residual stream / token shift / scalar-gain norm / windowed
+# attention with pooled far blocks (see _torch_ref.py for semantics).
+
+def scalar_rms_norm(x, gain, eps, out_dtype=None):
+    return get_backend(x.device).scalar_rms_norm(x, gain, eps, out_dtype)
+
+
+def add_scaled_scalar_norm(residual, y, gain, eps, mult, out_dtype=None):
+    return get_backend(residual.device).add_scaled_scalar_norm(
+        residual, y, gain, eps, mult, out_dtype)
+
+
+def token_shift(x, shift, state, state_rows, query_start_loc, out_dtype):
+    return get_backend(x.device).token_shift(
+        x, shift, state, state_rows, query_start_loc, out_dtype)
+
+
+def split_cache_write(key, value, k_cache, v_cache, slot_mapping):
+    return get_backend(key.device).split_cache_write(
+        key, value, k_cache, v_cache, slot_mapping)
+
+
+def pool_update(k_cache, v_cache, pool_k, pool_v, block_table,
+                query_start_loc, seq_lens, pool, max_query_len=0):
+    backend = get_backend(k_cache.device)
+    if backend is _torch_ref:
+        return backend.pool_update(k_cache, v_cache, pool_k, pool_v,
+                                   block_table, query_start_loc, seq_lens,
+                                   pool)
+    return backend.pool_update(k_cache, v_cache, pool_k, pool_v,
+                               block_table, query_start_loc, seq_lens,
+                               pool, max_query_len)
+
+
+def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
+                            block_table, query_start_loc, seq_lens, scale,
+                            window, pool, gate=None, num_decodes=0,
+                            max_seq_len=0, max_query_len=0):
+    return get_backend(q.device).pooled_window_attention(
+        q, k_cache, v_cache, pool_k, pool_v, block_table, query_start_loc,
+        seq_lens, scale, window, pool, gate, num_decodes, max_seq_len,
+        max_query_len)
+
+
+from vllm_amd.ops._torch_ref import pool_slots_per_page  # noqa: E402,F401

@@ -303,3 +303,155 @@ def grouped_topk(
         topk_weights = topk_weights / topk_weights.sum(-1, keepdim=True)
     topk_weights = topk_weights * routed_scaling_factor
     return topk_weights, topk_ids.to(torch.int32)
+
+
+# ---------------------------------------------------------------------
+# fp32 residual stream, token shift, scalar-gain RMS norm, and the
+# sliding-window attention with mean-pooled far blocks.
+
+def scalar_rms_norm(x, gain, eps, out_dtype=None):
+    """x / sqrt(mean(x^2) + eps) * gain with ONE gain for the whole row
+    (gain: 0-dim tensor). Math in fp32; result in out_dtype (fp32 when
+    None)."""
+    xf = x.float()
+    var = xf.pow(2).mean(dim=-1, keepdim=True)
+    out = xf / torch.sqrt(var + eps) * gain.float()
+    return out.to(out_dtype or torch.float32)
+
+
+def add_scaled_scalar_norm(residual, y, gain, eps, mult, out_dtype=None):
+    """residual += mult * scalar_rms_norm(y, gain), in place on the fp32
+    residual stream. Returns the updated residual, as a copy in
+    out_dtype when one is asked for (input of the next GEMM)."""
+    residual.add_(scalar_rms_norm(y, gain, eps), alpha=mult)
+    if out_dtype is None or out_dtype == residual.dtype:
+        return residual
+    return residual.to(out_dtype)
+
+
+def token_shift(x, shift, state, state_rows, query_start_loc, out_dtype):
+    """h[t] + (h[t-1] - h[t]) * shift per sequence; the token before a
+    chunk's first one comes from state[state_rows[r]] (zeros for a fresh
+    sequence), and the chunk's last h is stored back there. x: [T, W]
+    fp32; state: [rows, W] fp32 or None (no carry: zeros)."""
+    T = x.shape[0]
+    prev = torch.empty_like(x)
+    prev[1:] = x[:-1]
+    qs = query_start_loc.tolist()
+    for r in range(len(qs) - 1):
+        s, e = qs[r], qs[r + 1]
+        if s == e:
+            continue
+        if state is not None:
+            row = int(state_rows[r])
+            prev[s] = state[row]
+            state[row] = x[e - 1]
+        else:
+            prev[s] = 0
+    return (x + (prev - x) * shift.float()).to(out_dtype)
+
+
+def split_cache_write(key, value, k_cache, v_cache, slot_mapping):
+    """key [T, G, D] -> k_cache [blocks, G, block_size, D]; value
+    [T, G, Dv] -> v_cache [blocks, G, block_size, Dv] (key and value
+    widths may differ). Slots < 0 are skipped."""
+    block_size = k_cache.shape[2]
+    keep = slot_mapping >= 0
+    slots = slot_mapping[keep]
+    blk = slots // block_size
+    off = slots % block_size
+    k_cache[blk, :, off] = key[keep].to(k_cache.dtype)
+    v_cache[blk, :, off] = value[keep].to(v_cache.dtype)
+
+
+def _pool_slot(b, pool, block_size):
+    """Pooled block b (positions b*pool .. b*pool+pool-1) is stored with
+    the page that holds its LAST position; pages are block_size tokens.
+    Returns (logical page, slot inside that page's pooled area)."""
+    page = (b * pool + pool - 1) // block_size
+    return page, b - (page * block_size) // pool
+
+
+def pool_slots_per_page(pool, block_size):
+    return -(-block_size // pool)
+
+
+def pool_update(k_cache, v_cache, pool_k, pool_v, block_table,
+                query_start_loc, seq_lens, pool):
+    """Mean key/value of every pooled block that this step completed
+    (its last position was written this step), read back from the cache
+    as stored. pool_k/pool_v: [blocks, G, slots_per_page, D] fp32."""
+    bs = k_cache.shape[2]
+    qs = query_start_loc.tolist()
+    sl = seq_lens.tolist()
+    for r in range(len(sl)):
+        n = qs[r + 1] - qs[r]
+        end = sl[r]
+        start = end - n
+        # blocks whose last position b*pool + pool - 1 is in [start, end)
+        for b in range(start // pool, end // pool):
+            pos = torch.arange(b * pool, b * pool + pool,
+                               device=k_cache.device)
+            blk = block_table[r, pos // bs].long()
+            off = pos % bs
+            km = k_cache[blk, :, off].float().mean(0)   # [G, D]
+            vm = v_cache[blk, :, off].float().mean(0)
+            page, slot = _pool_slot(b, pool, bs)
+            pb = int(block_table[r, page])
+            pool_k[pb, :, slot] = km
+            pool_v[pb, :, slot] = vm
+
+
+def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
+                            block_table, query_start_loc, seq_lens, scale,
+                            window, pool, gate=None, num_decodes=0,
+                            max_seq_len=0, max_query_len=0):
+    """Position i attends the tokens j with 0 <= i - j < window plus one
+    pooled (mean) key/value per block of `pool` tokens that lies wholly
+    before the window (b*pool + pool - 1 <= i - window); one softmax
+    over both. gate: [T, H] logits — head outputs are multiplied by
+    sigmoid(gate). q: [T, H, D] -> [T, H, Dv]."""
+    T, H, D = q.shape
+    G = k_cache.shape[1]
+    Dv = v_cache.shape[3]
+    bs = k_cache.shape[2]
+    group = H // G
+    out = torch.empty(T, H, Dv, dtype=q.dtype, device=q.device)
+    qs = query_start_loc.tolist()
+    sl = seq_lens.tolist()
+    for r in range(len(sl)):
+        s, e = qs[r], qs[r + 1]
+        n = e - s
+        if n == 0:
+            continue
+        L = sl[r]
+        pos = torch.arange(L, device=q.device)
+        blk = block_table[r, pos // bs].long()
+        k_all = k_cache[blk, :, pos % bs].float()   # [L, G, D]
+        v_all = v_cache[blk, :, pos % bs].float()
+        nb_max = max(0, (L - 1 - window + 1) // pool)
+        if nb_max:
+            pk = torch.stack([
+                pool_k[int(block_table[r, _pool_slot(b, pool, bs)[0]]), :,
+                       _pool_slot(b, pool, bs)[1]] for b in range(nb_max)])
+            pv = torch.stack([
+                pool_v[int(block_table[r, _pool_slot(b, pool, bs)[0]]), :,
+                       _pool_slot(b, pool, bs)[1]] for b in range(nb_max)])
+        for t in range(n):
+            i = L - n + t
+            lo = max(0, i - window + 1)
+            nb = max(0, (i - window + 1) // pool)
+            kk = k_all[lo:i + 1]
+            vv = v_all[lo:i + 1]
+            if nb:
+                kk = torch.cat([pk[:nb].float(), kk])
+                vv = torch.cat([pv[:nb].float(), vv])
+            kk = kk.repeat_interleave(group, dim=1)   # [n, H, D]
+            vv = vv.repeat_interleave(group, dim=1)
+            sc = torch.einsum("hd,nhd->hn", q[s + t].float(), kk) * scale
+            p = torch.softmax(sc, dim=-1)
+            o = torch.einsum("hn,nhd->hd", p, vv)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[s + t].float()).unsqueeze(-1)
+            out[s + t] = o.to(out.dtype)
+    return out

@@ -53,6 +53,8 @@ class Request:
         mm_data: Optional[dict] = None,
         mm_hash: int = 0,
         encoder_tokens: int = 0,
+        prompt_open: bool = False,
+        logit_taps: Optional[list[int]] = None,
     ) -> None:
         self.request_id = request_id
         self.prompt_token_ids = prompt_token_ids
@@ -70,6 +72,14 @@ class Request:
         # (vision patches / audio frames / encoder prompt length);
         # metered by the scheduler's encoder admission budget.
         self.encoder_tokens = encoder_tokens
+
+        # Streamed prompt: while open, more prompt tokens may be
+        # appended (Scheduler.extend_prompt) and nothing is sampled at
+        # the end of the tokens seen so far.
+        self.prompt_open = prompt_open
+        # Absolute positions whose raw logits the client asked for; each
+        # is handed to the runner with the step that computes it.
+        self.logit_taps: list[int] = sorted(logit_taps or [])
 
         self.status = RequestStatus.WAITING
         self.stop_reason: Optional[object] = None
@@ -128,6 +138,22 @@ class Request:
         n = len(token_ids)
         self.num_tokens += n
         self.num_output_tokens += n
+
+    def extend_prompt(self, token_ids: list[int]) -> None:
+        assert self.prompt_open and not self.output_token_ids
+        self.prompt_token_ids.extend(token_ids)
+        self._all_token_ids.extend(token_ids)
+        self.num_tokens += len(token_ids)
+
+    def take_logit_taps(self, lo: int, hi: int) -> list[int]:
+        """Pending tap positions in [lo, hi), as offsets from lo."""
+        if not self.logit_taps:
+            return []
+        taken = [p - lo for p in self.logit_taps if lo <= p < hi]
+        if taken:
+            self.logit_taps = [p for p in self.logit_taps
+                               if not lo <= p < hi]
+        return taken
 
     def append_output_token(self, token_id: int) -> None:
         self.output_token_ids.append(token_id)

@@ -37,9 +37,10 @@ class AttentionMetadata:
     # kv_cache_coordinator.py:60). None = single-group model.
     block_table_w: Optional[torch.Tensor] = None
     slot_mapping_w: Optional[torch.Tensor] = None
-    # SSM (Mamba) models: per-request persistent state row indices, in
-    # this batch's request order (decodes first) — indexes the runner's
-    # conv/ssm state tensors. None for attention models.
+    # Models with per-request row state (SSM state, token-shift
+    # carry): persistent state row indices, in this batch's request
+    # order (decodes first) — indexes the runner's state tensors. None
+    # for models without such state.
     state_rows: Optional[torch.Tensor] = None
 
 
@@ -61,6 +62,10 @@ class ForwardContext:
     # ssm_states [L, rows, d_inner, d_state]) owned by the runner;
     # None for attention models and during memory profiling.
     mamba_states: Optional[tuple] = None
+    # Token-shift models: [layers, rows, width] fp32 — the previous
+    # token's mixer input per running request and layer, indexed by
+    # attn_metadata.state_rows; None during memory profiling.
+    shift_states: Optional[torch.Tensor] = None
     # Encoder-decoder (whisper): per-request cached audio-encoder
     # states, in this batch's request order ([T_audio, H] tensors or
     # None for requests without audio / padded rows).

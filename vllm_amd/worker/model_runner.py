@@ -46,6 +46,9 @@ class CachedReqState:
     block_ids_w: object = None    # window-group blocks (mixed models)
     mm_feats: object = None       # encoded-once projected patch rows
     mm_img_pos: object = None     # np positions of image tokens in prompt
+    # Streamed prompt: more prompt tokens may still arrive, so reaching
+    # the end of token_ids does not sample.
+    prompt_open: bool = False
 
     @property
     def output_token_ids(self) -> list[int]:
@@ -273,6 +276,11 @@ class ModelRunner:
         self.is_mamba = self.spec.has_mamba
         self.mamba_conv: Optional[torch.Tensor] = None
         self.mamba_ssm: Optional[torch.Tensor] = None
+        # Token-shift carry [layers, rows + 1, width] fp32 (same row
+        # discipline as the SSM state: one row per running request, a
+        # scratch row last, cleared on (re)admission).
+        self.has_row_state = self.spec.has_row_state
+        self.shift_states: Optional[torch.Tensor] = None
         self.np_block_table_w = (np.zeros((n, mb), dtype=np.int32)
                                  if self.mixed_attn else None)
         self.np_nblocks = np.zeros(n, dtype=np.int32)
@@ -428,6 +436,17 @@ class ModelRunner:
             # the profiled pool lands at a sane size (state tensors are
             # tiny and allocated separately in allocate_kv_cache).
             return self.block_size * 2 * spec.hidden_size * elt
+        if spec.layer_specs is not None:
+            # Per-layer geometry: K and V widths differ, and windowed
+            # layers with pooled far blocks add an fp32 pooled area.
+            total = 0
+            for entry in spec.layer_specs:
+                mx = entry["mixer"]
+                g, d, dv = mx["kv_heads"], mx["dim"], mx["vdim"]
+                total += self.block_size * g * (d + dv) * elt
+                slots = -(-self.block_size // int(mx["mask"]["pool"]))
+                total += slots * g * (d + dv) * 4
+            return total
         if spec.architecture == "jamba":
             kv_heads = spec.num_kv_heads_per_rank(get_tp_world_size())
             return (2 * self.block_size * kv_heads * spec.head_dim * elt
@@ -454,6 +473,37 @@ class ModelRunner:
             # encoded whole in one forward (chunking disabled). Blocks
             # remain admission accounting.
             self.kv_caches = []
+            self.graph_runner = None
+            return
+        if spec.has_token_shift:
+            rows = self.config.scheduler_config.max_num_seqs + 1
+            self.shift_states = torch.zeros(
+                spec.num_layers, rows, spec.hidden_size,
+                dtype=torch.float32, device=self.device)
+        if spec.layer_specs is not None:
+            # One (k, v, pooled k, pooled v) tuple per layer RUN — layers
+            # that borrow another layer's weights still cache their own
+            # keys. Head-major pages as for the other families; the
+            # pooled areas hold the finished block means in fp32.
+            from vllm_amd.ops import pool_slots_per_page
+            self.kv_caches = []
+            for entry in spec.layer_specs:
+                mx = entry["mixer"]
+                g, d, dv = mx["kv_heads"], mx["dim"], mx["vdim"]
+                slots = pool_slots_per_page(int(mx["mask"]["pool"]),
+                                            self.block_size)
+                self.kv_caches.append((
+                    torch.zeros(num_blocks, g, self.block_size, d,
+                                dtype=self.cache_dtype, device=self.device),
+                    torch.zeros(num_blocks, g, self.block_size, dv,
+                                dtype=self.cache_dtype, device=self.device),
+                    torch.zeros(num_blocks, g, slots, d,
+                                dtype=torch.float32, device=self.device),
+                    torch.zeros(num_blocks, g, slots, dv,
+                                dtype=torch.float32, device=self.device),
+                ))
+            # Decode stays eager: state rows are dynamic indices and the
+            # expert path may synchronize with the host.
             self.graph_runner = None
             return
         if spec.has_mamba:
@@ -701,6 +751,7 @@ class ModelRunner:
                 mm_data=nr.mm_data,
                 block_ids_w=(list(nr.block_ids_w)
                              if nr.block_ids_w is not None else None),
+                prompt_open=nr.prompt_open,
             )
             row = self._free_rows.pop()
             self._row_of[nr.req_id] = row
@@ -709,6 +760,8 @@ class ModelRunner:
                 # 0 (prefix caching is off for SSM models).
                 self.mamba_conv[:, row] = 0
                 self.mamba_ssm[:, row] = 0
+            if self.shift_states is not None:
+                self.shift_states[:, row] = 0
             nb = len(nr.block_ids)
             self.np_block_table[row, :nb] = nr.block_ids
             if self.mixed_attn and nr.block_ids_w:
@@ -717,18 +770,38 @@ class ModelRunner:
             self.np_nblocks[row] = nb
             self.np_computed[row] = nr.num_computed_tokens
             self.np_lora[row] = nr.lora_id
+            if nr.num_computed_tokens < len(nr.prompt_token_ids):
+                # A one-token step takes the decode path, which reads
+                # its input id from this row.
+                self.np_last_tok[row] = \
+                    nr.prompt_token_ids[nr.num_computed_tokens]
         cr = so.scheduled_cached_reqs
         for i, req_id in enumerate(cr.req_ids):
             state = self.requests[req_id]
             row = self._row_of[req_id]
             newb_w = (cr.new_block_ids_w[i]
                       if i < len(cr.new_block_ids_w) else None)
+            if state.prompt_open and not cr.resumed[i]:
+                # Streamed prompt: the scheduler sends the tokens this
+                # step runs; they are prompt, not sampled output.
+                nc = cr.num_computed_tokens[i]
+                del state.token_ids[nc:]
+                state.token_ids.extend(cr.new_token_ids[i])
+                state.prompt_len = len(state.token_ids)
+                if cr.new_token_ids[i]:
+                    self.np_last_tok[row] = cr.new_token_ids[i][-1]
+            if i < len(cr.prompt_open):
+                state.prompt_open = cr.prompt_open[i]
             if cr.resumed[i]:
                 if self.is_mamba and self.mamba_conv is not None:
                     self.mamba_conv[:, row] = 0
                     self.mamba_ssm[:, row] = 0
+                if self.shift_states is not None:
+                    self.shift_states[:, row] = 0
                 state.block_ids = list(cr.new_block_ids[i])
                 state.token_ids = list(cr.new_token_ids[i])
+                if state.prompt_open:
+                    state.prompt_len = len(state.token_ids)
                 state.num_computed_tokens = cr.num_computed_tokens[i]
                 nb = len(state.block_ids)
                 self.np_block_table[row, :nb] = state.block_ids
@@ -751,6 +824,11 @@ class ModelRunner:
                     state.block_ids_w.extend(newb_w)
                     self.np_block_table_w[row, w0:w0 + len(newb_w)] = newb_w
             self.np_computed[row] = cr.num_computed_tokens[i]
+            nc = cr.num_computed_tokens[i]
+            if nc < len(state.token_ids):
+                # Known next input (rest of a prompt): the decode path
+                # reads it from the row when the step has one token.
+                self.np_last_tok[row] = state.token_ids[nc]
 
     # ------------------------------------------------------------------
     @torch.inference_mode()
@@ -774,7 +852,7 @@ class ModelRunner:
         padded entries land on the scratch row (last)."""
         sr = rows
         if np_pad:
-            scratch = self.mamba_conv.shape[1] - 1
+            scratch = self.config.scheduler_config.max_num_seqs
             sr = np.concatenate(
                 [sr, np.full(np_pad, scratch, dtype=np.int64)])
         return torch.from_numpy(np.ascontiguousarray(sr)).to(dev)
@@ -800,6 +878,12 @@ class ModelRunner:
             cur = self._row_pos[rows]
             self._row_pos[last_rows] = -1
             hit = cur >= 0
+            # Rows still inside their prompt feed the known prompt
+            # token, not a sampled one.
+            for j, r in enumerate(req_ids):
+                st = self.requests[r]
+                if st.num_computed_tokens < len(st.token_ids):
+                    hit[j] = False
             if hit.all():
                 idx = torch.from_numpy(cur).to(last_t.device)
                 ids_dev = last_t.index_select(0, idx)
@@ -897,7 +981,7 @@ class ModelRunner:
                 slot_mapping_w=(torch.from_numpy(slot_mapping_w).to(dev)
                                 if slot_mapping_w is not None else None),
                 state_rows=(self._state_rows(rows, np_pad, dev)
-                            if self.is_mamba else None),
+                            if self.has_row_state else None),
             )
             ids_t = (ids_dev if ids_dev is not None
                      else torch.from_numpy(input_ids).to(dev))
@@ -916,6 +1000,7 @@ class ModelRunner:
                 sp_size=self.sp_size,
                 mamba_states=((self.mamba_conv, self.mamba_ssm)
                               if self.is_mamba else None),
+                shift_states=self.shift_states,
                 cross_feats=cross,
             )
             with set_forward_context(ctx):
@@ -925,13 +1010,39 @@ class ModelRunner:
 
         self.np_computed[rows] += 1
         states = [self.requests[r] for r in req_ids]
+        # Rows that do not sample: the step ended inside the prompt, or
+        # the prompt is streamed and still open.
+        silent = [j for j, st in enumerate(states)
+                  if st.prompt_open
+                  or st.num_computed_tokens + 1 < len(st.token_ids)]
         for st in states:
             st.num_computed_tokens += 1
+        tapped = None
+        if so.logit_taps:
+            tapped = {r: logits[j:j + 1].float().cpu()
+                      for j, r in enumerate(req_ids)
+                      if so.logit_taps.get(r)}
+        if len(silent) == n:
+            self._last_sampled = None
+            out = ModelRunnerOutput(
+                req_ids=req_ids, sampled_token_ids=[[] for _ in req_ids],
+                tapped_logits=tapped)
+            return AsyncModelOutput(lambda: out)
 
         s_meta = self._sampling_meta(req_ids, states, dev)
         s_meta = self._with_grammar_masks(s_meta, states)
         s_out = self.sampler(logits, s_meta)
         sampled_t = s_out.sampled_token_ids
+        if silent:
+            keep = np.setdiff1d(np.arange(n), np.asarray(silent))
+            self._last_sampled = (
+                sampled_t[torch.from_numpy(keep).to(sampled_t.device)],
+                rows[keep])
+            sampled_np = sampled_t.cpu().numpy()
+            out = self._finish_decode(req_ids, states, rows, sampled_np,
+                                      s_out.logprobs, None, silent=silent)
+            out.tapped_logits = tapped
+            return AsyncModelOutput(lambda: out)
         self._last_sampled = (sampled_t, rows)
 
         draft_map = None
@@ -972,14 +1083,17 @@ class ModelRunner:
             def finish() -> ModelRunnerOutput:
                 ev.synchronize()
                 sampled_np = pin[:n].numpy().copy()
-                return self._finish_decode(req_ids, states, rows, sampled_np,
-                                           None, draft_map)
+                res = self._finish_decode(req_ids, states, rows, sampled_np,
+                                          None, draft_map)
+                res.tapped_logits = tapped
+                return res
 
             return AsyncModelOutput(finish)
 
         sampled_np = sampled_t.cpu().numpy()
         out = self._finish_decode(req_ids, states, rows, sampled_np,
                                   s_out.logprobs, draft_map)
+        out.tapped_logits = tapped
         return AsyncModelOutput(lambda: out)
 
     def _with_grammar_masks(self, meta, states):
@@ -994,12 +1108,24 @@ class ModelRunner:
         return meta
 
     def _finish_decode(self, req_ids, states, rows, sampled_np,
-                       logprobs, draft_map=None) -> ModelRunnerOutput:
-        self.np_last_tok[rows] = sampled_np
+                       logprobs, draft_map=None,
+                       silent=None) -> ModelRunnerOutput:
         sampled = sampled_np.tolist()
         sampled_per_req = [[int(t)] for t in sampled]
+        if silent:
+            mute = set(silent)
+            live = np.asarray([j for j in range(len(rows))
+                               if j not in mute], dtype=np.int64)
+            self.np_last_tok[rows[live]] = sampled_np[live]
+            for j in silent:
+                sampled_per_req[j] = []
+        else:
+            mute = ()
+            self.np_last_tok[rows] = sampled_np
         logprobs_per_req: dict[str, list[dict[int, float]]] = {}
         for j, st in enumerate(states):
+            if j in mute:
+                continue
             if st.grammar is not None and st.grammar_state is not None:
                 st.grammar_state = st.grammar.advance(
                     st.grammar_state, int(sampled[j]))
@@ -1129,7 +1255,8 @@ class ModelRunner:
                 sampling_npos.append(len(spec_map[rid]) + 1)
             elif state.sampling_params.pooling:
                 pooling_rows.append((rid, i, n, start))
-            elif start + n >= len(state.token_ids):
+            elif (start + n >= len(state.token_ids)
+                    and not state.prompt_open):
                 sampling_rows.append(i)
                 sampling_npos.append(1)
             if (state.sampling_params.prompt_logprobs
@@ -1159,7 +1286,7 @@ class ModelRunner:
             state_rows=(torch.tensor(
                 [self._row_of[rid] for rid, _ in items],
                 dtype=torch.int64, device=dev)
-                if self.is_mamba else None),
+                if self.has_row_state else None),
         )
         input_ids_t = torch.from_numpy(input_ids).to(dev)
         positions_t = torch.from_numpy(positions).to(dev)
@@ -1231,6 +1358,7 @@ class ModelRunner:
             mm_embeds=mm_embeds,
             mamba_states=((self.mamba_conv, self.mamba_ssm)
                           if self.is_mamba else None),
+            shift_states=self.shift_states,
             cross_feats=cross_feats,
         )
         if self.pp_size > 1:
@@ -1259,6 +1387,22 @@ class ModelRunner:
         for rid, n in items:
             self.requests[rid].num_computed_tokens += n
             self.np_computed[self._row_of[rid]] += n
+
+        tapped_map = None
+        if so.logit_taps:
+            rows_of = {rid: i for i, (rid, _n) in enumerate(items)}
+            tap_idx: list[int] = []
+            tap_cnt: list[tuple[str, int]] = []
+            for rid, offs in so.logit_taps.items():
+                base = int(query_start_loc[rows_of[rid]])
+                tap_idx.extend(base + o for o in offs)
+                tap_cnt.append((rid, len(offs)))
+            tap_logits = self.model.compute_logits(
+                hidden[torch.tensor(tap_idx, device=dev)]).float().cpu()
+            tapped_map, at = {}, 0
+            for rid, c in tap_cnt:
+                tapped_map[rid] = tap_logits[at:at + c]
+                at += c
 
         plp_map: dict[str, list[dict[int, float]]] = {}
         for rid, i, n, start in plp_rows:
@@ -1319,6 +1463,7 @@ class ModelRunner:
                 sampled_token_ids=[[] for _ in req_ids],
                 pooled=pooled_map or None,
                 prompt_logprobs=plp_map or None,
+                tapped_logits=tapped_map,
             )
 
         if self.pp_size > 1:
@@ -1521,6 +1666,7 @@ class ModelRunner:
             draft_token_ids=draft_map,
             pooled=pooled_map or None,
             prompt_logprobs=plp_map or None,
+            tapped_logits=tapped_map,
         )
 
     # ------------------------------------------------------------------
