@@ -28,6 +28,8 @@ SOURCES = [
     CSRC / "quant_fp8.hip",
     CSRC / "attention_decode.hip",
     CSRC / "attention_prefill.hip",
+    CSRC / "pooled_attention.hip",
+    CSRC / "pooled_attention_prefill.hip",
     CSRC / "gemm_hipblaslt.cpp",
     CSRC / "bindings.cpp",
 ]
@@ -53,6 +55,8 @@ def _torch_flags() -> tuple[list[str], list[str]]:
         f"--offload-arch={ARCH}",
         "-fno-gpu-rdc",
         "-Wno-unused-result",
+        # Keep packed-fp32 VALU forms out of the generated code.
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     ]
     link = [
         f"-L{torch_dir}/lib",
@@ -73,29 +77,45 @@ def needs_build() -> bool:
     if not OUT_SO.exists():
         return True
     so_mtime = OUT_SO.stat().st_mtime
-    deps = list(SOURCES) + [CSRC / "common.h", Path(__file__)]
+    deps = list(SOURCES) + [CSRC / "common.h",
+                            CSRC / "pooled_attention.h", Path(__file__)]
     return any(p.stat().st_mtime > so_mtime for p in deps)
 
 
 def build(verbose: bool = True) -> Path:
     flags, link = _torch_flags()
+    from concurrent.futures import ThreadPoolExecutor
+
     objs = []
     build_dir = CSRC / ".build"
     build_dir.mkdir(exist_ok=True)
+    cmds = []
     for src in SOURCES:
         obj = build_dir / (src.stem + ".o")
         cmd = [HIPCC, "-c", str(src), "-o", str(obj)] + flags
         if src.suffix == ".hip":
             cmd.insert(1, "-x")
             cmd.insert(2, "hip")
+        cmds.append(cmd)
+        objs.append(str(obj))
+
+    def compile_one(cmd):
         if verbose:
             print("[vllm_amd.build]", " ".join(cmd), file=sys.stderr)
-        subprocess.run(cmd, check=True)
-        objs.append(str(obj))
+        # Build chatter never goes to stdout: callers may speak a
+        # line protocol there.
+        subprocess.run(cmd, check=True, stdout=sys.stderr)
+
+    # One translation unit per core: the files are independent and the
+    # slowest one bounds the wall time.
+    jobs = int(os.environ.get("MAX_JOBS", "0")) or min(
+        len(cmds), os.cpu_count() or 4)
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        list(pool.map(compile_one, cmds))
     cmd = [HIPCC, "-shared", "-o", str(OUT_SO)] + objs + link
     if verbose:
         print("[vllm_amd.build]", " ".join(cmd), file=sys.stderr)
-    subprocess.run(cmd, check=True)
+    subprocess.run(cmd, check=True, stdout=sys.stderr)
     return OUT_SO
 
 

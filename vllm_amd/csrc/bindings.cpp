@@ -55,6 +55,40 @@ void mla_decode(torch::Tensor out, torch::Tensor q_nope, torch::Tensor q_pe,
                 torch::Tensor kv_cache, torch::Tensor block_table,
                 torch::Tensor seq_lens, double scale, int64_t max_seq_len,
                 torch::Tensor tmp_out, torch::Tensor tmp_lse);
+torch::Tensor scalar_rms_norm(torch::Tensor x, torch::Tensor gain,
+                              double eps, torch::ScalarType out_dtype);
+torch::Tensor add_scaled_scalar_norm(
+    torch::Tensor residual, torch::Tensor y, torch::Tensor gain, double eps,
+    double mult, c10::optional<torch::ScalarType> out_dtype);
+torch::Tensor token_shift(torch::Tensor x, torch::Tensor mu,
+                          c10::optional<torch::Tensor> state,
+                          c10::optional<torch::Tensor> state_rows,
+                          torch::Tensor query_start_loc,
+                          torch::ScalarType out_dtype);
+torch::Tensor silu_and_mul_any(torch::Tensor x);
+torch::Tensor norm_qk_cache_write(torch::Tensor q, torch::Tensor k,
+                                  torch::Tensor v,
+                                  c10::optional<torch::Tensor> q_w,
+                                  c10::optional<torch::Tensor> k_w, double eps,
+                                  torch::Tensor k_cache, torch::Tensor v_cache,
+                                  torch::Tensor slot_mapping);
+void pool_update(torch::Tensor k_cache, torch::Tensor v_cache,
+                 torch::Tensor pool_k, torch::Tensor pool_v,
+                 torch::Tensor block_table, torch::Tensor query_start_loc,
+                 torch::Tensor seq_lens, int64_t pool, int64_t max_query_len);
+void pooled_window_attention_rows(
+    torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+    torch::Tensor v_cache, torch::Tensor pool_k, torch::Tensor pool_v,
+    torch::Tensor block_table, torch::Tensor query_start_loc,
+    torch::Tensor seq_lens, c10::optional<torch::Tensor> gate, double scale,
+    int64_t window, int64_t pool, int64_t row0, int64_t num_rows);
+void pooled_window_attention_prefill(
+    torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+    torch::Tensor v_cache, torch::Tensor pool_k, torch::Tensor pool_v,
+    torch::Tensor block_table, torch::Tensor query_start_loc,
+    torch::Tensor seq_lens, c10::optional<torch::Tensor> gate, double scale,
+    int64_t window, int64_t pool, int64_t num_decodes,
+    int64_t max_query_len);
 torch::Tensor car_init(int64_t rank, int64_t world, int64_t max_bytes);
 void car_connect(torch::Tensor handles);
 bool car_is_ready();
@@ -104,6 +138,30 @@ TORCH_LIBRARY(vllm_amd, m) {
         "Tensor kv_cache, Tensor block_table, Tensor seq_lens, "
         "float scale, int max_seq_len, Tensor(b!) tmp_out, "
         "Tensor(c!) tmp_lse) -> ()");
+  m.def("scalar_rms_norm(Tensor x, Tensor gain, float eps, "
+        "ScalarType out_dtype) -> Tensor");
+  m.def("add_scaled_scalar_norm(Tensor(a!) residual, Tensor y, Tensor gain, "
+        "float eps, float mult, ScalarType? out_dtype) -> Tensor");
+  m.def("token_shift(Tensor x, Tensor mu, Tensor(a!)? state, "
+        "Tensor? state_rows, Tensor query_start_loc, ScalarType out_dtype)"
+        " -> Tensor");
+  m.def("silu_and_mul_any(Tensor x) -> Tensor");
+  m.def("norm_qk_cache_write(Tensor q, Tensor k, Tensor v, Tensor? q_w, "
+        "Tensor? k_w, float eps, Tensor(a!) k_cache, Tensor(b!) v_cache, "
+        "Tensor slot_mapping) -> Tensor");
+  m.def("pool_update(Tensor k_cache, Tensor v_cache, Tensor(a!) pool_k, "
+        "Tensor(b!) pool_v, Tensor block_table, Tensor query_start_loc, "
+        "Tensor seq_lens, int pool, int max_query_len) -> ()");
+  m.def("pooled_window_attention_rows(Tensor(a!) out, Tensor q, "
+        "Tensor k_cache, Tensor v_cache, Tensor pool_k, Tensor pool_v, "
+        "Tensor block_table, Tensor query_start_loc, Tensor seq_lens, "
+        "Tensor? gate, float scale, int window, int pool, int row0, "
+        "int num_rows) -> ()");
+  m.def("pooled_window_attention_prefill(Tensor(a!) out, Tensor q, "
+        "Tensor k_cache, Tensor v_cache, Tensor pool_k, Tensor pool_v, "
+        "Tensor block_table, Tensor query_start_loc, Tensor seq_lens, "
+        "Tensor? gate, float scale, int window, int pool, int num_decodes, "
+        "int max_query_len) -> ()");
   // Custom xGMI collectives (comms.hip). init/connect/destroy are
   // host-side control ops and live on the catch-all dispatch below.
   m.def("car_init(int rank, int world, int max_bytes) -> Tensor");
@@ -144,4 +202,14 @@ TORCH_LIBRARY_IMPL(vllm_amd, CUDA, m) {
   m.impl("moe_gemm_shuf", &vllm_amd::moe_gemm_shuf);
   m.impl("moe_combine", &vllm_amd::moe_combine);
   m.impl("mla_decode", &vllm_amd::mla_decode);
+  m.impl("scalar_rms_norm", &vllm_amd::scalar_rms_norm);
+  m.impl("add_scaled_scalar_norm", &vllm_amd::add_scaled_scalar_norm);
+  m.impl("token_shift", &vllm_amd::token_shift);
+  m.impl("silu_and_mul_any", &vllm_amd::silu_and_mul_any);
+  m.impl("norm_qk_cache_write", &vllm_amd::norm_qk_cache_write);
+  m.impl("pool_update", &vllm_amd::pool_update);
+  m.impl("pooled_window_attention_prefill",
+         &vllm_amd::pooled_window_attention_prefill);
+  m.impl("pooled_window_attention_rows",
+         &vllm_amd::pooled_window_attention_rows);
 }

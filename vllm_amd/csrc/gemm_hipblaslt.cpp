@@ -177,7 +177,14 @@ void run_matmul(torch::Tensor& out, const torch::Tensor& a,
   TORCH_CHECK(w.size(1) == K && out.size(0) == M && out.size(1) == N);
   TORCH_CHECK(a.is_contiguous() && w.is_contiguous() && out.is_contiguous());
   const bool is_bf16 = a.scalar_type() == torch::kBFloat16;
-  hipDataType dt = is_bf16 ? HIP_R_16BF : HIP_R_16F;
+  const bool is_f32 = a.scalar_type() == torch::kFloat32;
+  TORCH_CHECK(is_bf16 || is_f32 || a.scalar_type() == torch::kHalf,
+              "lt_linear: bf16, fp16 or fp32 operands");
+  TORCH_CHECK(w.scalar_type() == a.scalar_type() &&
+              out.scalar_type() == a.scalar_type());
+  // fp32 operands run true fp32 (COMPUTE_32F, no reduced-precision
+  // matrix mode).
+  hipDataType dt = is_f32 ? HIP_R_32F : (is_bf16 ? HIP_R_16BF : HIP_R_16F);
 
   auto& c = ctx();
   auto stream = c10::hip::getCurrentHIPStream().stream();
@@ -208,7 +215,8 @@ void run_matmul(torch::Tensor& out, const torch::Tensor& a,
   HIPBLASLT_CHECK(hipblasLtMatrixLayoutCreate(&lc, dt, N, M, N));
 
   const float alpha = 1.f, beta = 0.f;
-  const uint64_t key = shape_key(M, N, K, is_bf16, has_bias);
+  const uint64_t key = shape_key(M, N, K, is_bf16, has_bias) ^
+                       (is_f32 ? (1ull << 63) : 0ull);
 
   auto call = [&](const hipblasLtMatmulAlgo_t& cand) {
     return hipblasLtMatmul(

@@ -133,17 +133,21 @@ class PooledWindowAttention(nn.Module):
         self.window = window
         self.pool = pool
 
-    def forward(self, q, k, v, gate, cache_idx: int) -> torch.Tensor:
+    def forward(self, q, k, v, gate, cache_idx: int,
+                qk_norm=None) -> torch.Tensor:
         """q [T, H, D], k [T, G, D], v [T, G, Dv], gate [T, H] or None
         (all may be strided slices of one fused projection) ->
-        [T, H * Dv]."""
+        [T, H * Dv]. qk_norm = (q_weight [D], k_weight [D], eps) applies
+        a per-head RMS norm to q and k inside the cache-write pass."""
         ctx = get_forward_context()
         meta = ctx.attn_metadata
         T = q.shape[0]
         if not ctx.kv_caches:
             return self._profile_attention(q, k, v, gate, meta)
         k_cache, v_cache, pool_k, pool_v = ctx.kv_caches[cache_idx]
-        ops.split_cache_write(k, v, k_cache, v_cache, meta.slot_mapping)
+        q_w, k_w, eps = qk_norm if qk_norm is not None else (None, None, 0.0)
+        q = ops.norm_qk_cache_write(q, k, v, q_w, k_w, eps, k_cache,
+                                    v_cache, meta.slot_mapping)
         ops.pool_update(k_cache, v_cache, pool_k, pool_v, meta.block_table,
                         meta.query_start_loc, meta.seq_lens, self.pool,
                         max_query_len=meta.max_query_len)

@@ -82,13 +82,13 @@ class GadilixAttentionMixer(nn.Module):
         a = self.q_size
         b = a + self.k_size
         c = b + self.v_size
-        q = qkvg[:, :a].reshape(T * self.H, self.D)
-        k = qkvg[:, a:b].reshape(T * self.G, self.D)
-        q = self.q_norm(q.contiguous()).view(T, self.H, self.D)
-        k = self.k_norm(k.contiguous()).view(T, self.G, self.D)
+        q = qkvg[:, :a].view(T, self.H, self.D)
+        k = qkvg[:, a:b].view(T, self.G, self.D)
         v = qkvg[:, b:c].view(T, self.G, self.Dv)
         gate = qkvg[:, c:c + self.H]
-        out = self.attn(q, k, v, gate, cache_idx)
+        out = self.attn(q, k, v, gate, cache_idx,
+                        qk_norm=(self.q_norm.weight, self.k_norm.weight,
+                                 self.q_norm.eps))
         return self.o_proj(out)
 
     def load_fused(self, q, k, v, g) -> None:

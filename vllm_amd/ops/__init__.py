@@ -194,6 +194,12 @@ def split_cache_write(key, value, k_cache, v_cache, slot_mapping):
         key, value, k_cache, v_cache, slot_mapping)
 
 
+def norm_qk_cache_write(q, k, v, q_w, k_w, eps, k_cache, v_cache,
+                        slot_mapping):
+    return get_backend(q.device).norm_qk_cache_write(
+        q, k, v, q_w, k_w, eps, k_cache, v_cache, slot_mapping)
+
+
 def pool_update(k_cache, v_cache, pool_k, pool_v, block_table,
                 query_start_loc, seq_lens, pool, max_query_len=0):
     backend = get_backend(k_cache.device)

@@ -364,6 +364,18 @@ def split_cache_write(key, value, k_cache, v_cache, slot_mapping):
     v_cache[blk, :, off] = value[keep].to(v_cache.dtype)
 
 
+def norm_qk_cache_write(q, k, v, q_w, k_w, eps, k_cache, v_cache,
+                        slot_mapping):
+    """Per-head RMS norm of q and k (weights [D] shared by all heads;
+    None = no norm), then the paged K/V write. Returns the normed q
+    [T, H, D], contiguous."""
+    if q_w is not None:
+        q = rms_norm(q.reshape(-1, q.shape[-1]), q_w, eps).view(q.shape)
+        k = rms_norm(k.reshape(-1, k.shape[-1]), k_w, eps).view(k.shape)
+    split_cache_write(k, v, k_cache, v_cache, slot_mapping)
+    return q.contiguous()
+
+
 def _pool_slot(b, pool, block_size):
     """Pooled block b (positions b*pool .. b*pool+pool-1) is stored with
     the page that holds its LAST position; pages are block_size tokens.

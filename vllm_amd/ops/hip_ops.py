@@ -43,6 +43,13 @@ def apply_rope(positions, q, k, cos_sin_cache, rotary_dim, is_neox=True):
 
 
 def silu_and_mul(x):
+    if x.dtype == torch.float32:
+        # The 16-bit kernel above is vectorized for 2-byte elements;
+        # fp32 rows take the generic one.
+        shape = list(x.shape)
+        out = _C.silu_and_mul_any(x.reshape(-1, shape[-1]).contiguous())
+        shape[-1] //= 2
+        return out.reshape(shape)
     return _C.silu_and_mul(x)
 
 
@@ -332,3 +339,77 @@ def fused_moe(hidden, w13, w2, topk_weights, topk_ids, activation="silu",
     out = torch.zeros(T, H, dtype=torch.float32, device=hidden.device)
     out.index_add_(0, token_of, out_sorted.float() * w)
     return out.to(hidden.dtype)
+
+
+# ---------------------------------------------------------------------
+# fp32 residual stream / token shift / scalar-gain norm / windowed
+# attention with pooled far blocks (csrc/pooled_attention*.hip).
+
+def scalar_rms_norm(x, gain, eps, out_dtype=None):
+    return _C.scalar_rms_norm(x.contiguous(), gain, eps,
+                              out_dtype or torch.float32)
+
+
+def add_scaled_scalar_norm(residual, y, gain, eps, mult, out_dtype=None):
+    return _C.add_scaled_scalar_norm(residual, y.contiguous(), gain, eps,
+                                     mult, out_dtype)
+
+
+def token_shift(x, shift, state, state_rows, query_start_loc, out_dtype):
+    return _C.token_shift(x, shift, state,
+                          state_rows if state is not None else None,
+                          query_start_loc, out_dtype)
+
+
+def norm_qk_cache_write(q, k, v, q_w, k_w, eps, k_cache, v_cache,
+                        slot_mapping):
+    return _C.norm_qk_cache_write(q, k, v, q_w, k_w, eps, k_cache, v_cache,
+                                  slot_mapping)
+
+
+def split_cache_write(key, value, k_cache, v_cache, slot_mapping):
+    # Same kernel without norms; the normed-q output is unused here.
+    _C.norm_qk_cache_write(key[:, :0], key, value, None, None, 0.0,
+                           k_cache, v_cache, slot_mapping)
+
+
+def pool_update(k_cache, v_cache, pool_k, pool_v, block_table,
+                query_start_loc, seq_lens, pool, max_query_len=0):
+    if max_query_len <= 0:
+        qsl = query_start_loc
+        max_query_len = int((qsl[1:] - qsl[:-1]).max().item())
+    _C.pool_update(k_cache, v_cache, pool_k, pool_v, block_table,
+                   query_start_loc, seq_lens, pool, max_query_len)
+
+
+def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
+                            block_table, query_start_loc, seq_lens, scale,
+                            window, pool, gate=None, num_decodes=0,
+                            max_seq_len=0, max_query_len=0):
+    """Decode rows (the first num_decodes requests, one token each) run
+    on the row-wise kernel; prefill chunks run on the MFMA tile kernel
+    in bf16 and on the row-wise kernel in fp16/fp32."""
+    import os
+
+    T, H, _ = q.shape
+    q = q.contiguous()
+    out = torch.empty(T, H, v_cache.shape[3], dtype=q.dtype,
+                      device=q.device)
+    num_reqs = seq_lens.shape[0]
+    tiled = (q.dtype == torch.bfloat16
+             and os.environ.get("VLLM_AMD_PWA_ROWWISE", "0") != "1")
+    n_rows = T if not tiled else num_decodes
+    if n_rows > 0:
+        _C.pooled_window_attention_rows(
+            out, q, k_cache, v_cache, pool_k, pool_v, block_table,
+            query_start_loc, seq_lens, gate, scale, window, pool, 0,
+            n_rows)
+    if tiled and num_decodes < num_reqs:
+        if max_query_len <= 0:
+            qsl = query_start_loc
+            max_query_len = int((qsl[1:] - qsl[:-1]).max().item())
+        _C.pooled_window_attention_prefill(
+            out, q, k_cache, v_cache, pool_k, pool_v, block_table,
+            query_start_loc, seq_lens, gate, scale, window, pool,
+            num_decodes, max_query_len)
+    return out
