@@ -58,7 +58,12 @@ def gelu_and_mul(x):
 
 
 def linear(x, weight, bias=None):
-    # Tuned hipBLASLt GEMM (per-shape algo search on first use).
+    # Tuned hipBLASLt GEMM (per-shape algo search on first use). Rows
+    # that are not 16-byte multiples fall outside its aligned kernels:
+    # those shapes go to torch's vendor GEMM instead.
+    per16 = 4 if x.dtype == torch.float32 else 8
+    if weight.shape[0] % per16 or weight.shape[1] % per16:
+        return torch.nn.functional.linear(x, weight, bias)
     return _C.lt_linear(x, weight, bias)
 
 
