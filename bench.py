@@ -58,11 +58,26 @@ def parse_args():
                         "replica per rank, each with its own --batch (weak "
                         "scaling, xGMI-free — the throughput-optimal "
                         "serving layout for an 8B model)")
+    p.add_argument("--compare-family", type=str, default=None,
+                   choices=["gadilix"],
+                   help="instead of the flagship workload: prefill and "
+                        "decode throughput of this family beside the "
+                        "closest existing one at equal active size "
+                        "(benchmarks/family_compare.py; one JSON line "
+                        "per family, size and phase)")
+    p.add_argument("--compare-sizes", type=str, default="small,medium")
+    p.add_argument("--compare-prompt-len", type=int, default=4096)
     return p.parse_args()
 
 
 def main():
     args = parse_args()
+    if args.compare_family:
+        from benchmarks.family_compare import main as compare
+
+        compare(args.compare_family, args.compare_sizes,
+                prompt_len=args.compare_prompt_len)
+        return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     local_rank = int(os.environ.get("LOCAL_RANK", str(rank)))

@@ -418,6 +418,10 @@ def test_moe_grouped_gemm_kernel(T, H, I, E, K):
     assert_close(out, expect, atol=8e-2, rtol=8e-2)
 
 
+# Captured under inference mode like the engine's own captures: the
+# default CUDA generator's capture state may have been created by an
+# earlier inference-mode step, and capture_begin updates it in place.
+@torch.inference_mode()
 def test_moe_hip_graph_capturable():
     """The grouped-GEMM path must capture and replay in a hipGraph with
     correct results (static shapes, no host syncs)."""

@@ -50,6 +50,10 @@ def test_world1_collectives_identity():
 
 
 @pytest.mark.gpu
+# Captured under inference mode like the engine's own captures: the
+# default CUDA generator's capture state may have been created by an
+# earlier inference-mode step, and capture_begin updates it in place.
+@torch.inference_mode()
 def test_world1_graph_capturable():
     """The point of the direct binding: collectives captured in a
     hipGraph replay correctly."""

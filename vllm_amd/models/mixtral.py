@@ -46,6 +46,8 @@ class MixtralAttention(nn.Module):
         self.attn = Attention(
             self.num_heads, spec.head_dim, scale=spec.head_dim**-0.5,
             num_kv_heads=self.num_kv_heads, layer_idx=layer_idx,
+            # Mistral-style uniform window when the spec sets one.
+            sliding_window=spec.sliding_window,
         )
 
     def forward(self, positions, hidden):
