@@ -30,6 +30,7 @@ SOURCES = [
     CSRC / "attention_prefill.hip",
     CSRC / "pooled_attention.hip",
     CSRC / "pooled_attention_prefill.hip",
+    CSRC / "pooled_attention_decode.hip",
     CSRC / "gemm_hipblaslt.cpp",
     CSRC / "bindings.cpp",
 ]

@@ -89,6 +89,12 @@ void pooled_window_attention_prefill(
     torch::Tensor seq_lens, c10::optional<torch::Tensor> gate, double scale,
     int64_t window, int64_t pool, int64_t num_decodes,
     int64_t max_query_len);
+void pooled_window_attention_decode(
+    torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+    torch::Tensor v_cache, torch::Tensor pool_k, torch::Tensor pool_v,
+    torch::Tensor block_table, torch::Tensor query_start_loc,
+    torch::Tensor seq_lens, c10::optional<torch::Tensor> gate, double scale,
+    int64_t window, int64_t pool, int64_t num_decodes, int64_t max_seq_len);
 torch::Tensor car_init(int64_t rank, int64_t world, int64_t max_bytes);
 void car_connect(torch::Tensor handles);
 bool car_is_ready();
@@ -162,6 +168,11 @@ TORCH_LIBRARY(vllm_amd, m) {
         "Tensor block_table, Tensor query_start_loc, Tensor seq_lens, "
         "Tensor? gate, float scale, int window, int pool, int num_decodes, "
         "int max_query_len) -> ()");
+  m.def("pooled_window_attention_decode(Tensor(a!) out, Tensor q, "
+        "Tensor k_cache, Tensor v_cache, Tensor pool_k, Tensor pool_v, "
+        "Tensor block_table, Tensor query_start_loc, Tensor seq_lens, "
+        "Tensor? gate, float scale, int window, int pool, int num_decodes, "
+        "int max_seq_len) -> ()");
   // Custom xGMI collectives (comms.hip). init/connect/destroy are
   // host-side control ops and live on the catch-all dispatch below.
   m.def("car_init(int rank, int world, int max_bytes) -> Tensor");
@@ -212,4 +223,6 @@ TORCH_LIBRARY_IMPL(vllm_amd, CUDA, m) {
          &vllm_amd::pooled_window_attention_prefill);
   m.impl("pooled_window_attention_rows",
          &vllm_amd::pooled_window_attention_rows);
+  m.impl("pooled_window_attention_decode",
+         &vllm_amd::pooled_window_attention_decode);
 }

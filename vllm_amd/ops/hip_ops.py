@@ -392,8 +392,9 @@ def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
                             window, pool, gate=None, num_decodes=0,
                             max_seq_len=0, max_query_len=0):
     """Decode rows (the first num_decodes requests, one token each) run
-    on the row-wise kernel; prefill chunks run on the MFMA tile kernel
-    in bf16 and on the row-wise kernel in fp16/fp32."""
+    on the split-key decode kernel in 16-bit dtypes; prefill chunks run
+    on the MFMA tile kernel in bf16. fp32 (and fp16 prefill rows) use
+    the row-wise kernel, which VLLM_AMD_PWA_ROWWISE=1 forces for all."""
     import os
 
     T, H, _ = q.shape
@@ -401,13 +402,23 @@ def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
     out = torch.empty(T, H, v_cache.shape[3], dtype=q.dtype,
                       device=q.device)
     num_reqs = seq_lens.shape[0]
-    tiled = (q.dtype == torch.bfloat16
-             and os.environ.get("VLLM_AMD_PWA_ROWWISE", "0") != "1")
-    n_rows = T if not tiled else num_decodes
+    rowwise = os.environ.get("VLLM_AMD_PWA_ROWWISE", "0") == "1"
+    half = q.dtype in (torch.bfloat16, torch.float16) and not rowwise
+    tiled = q.dtype == torch.bfloat16 and not rowwise
+    row0 = 0
+    if half and num_decodes > 0:
+        if max_seq_len <= 0:
+            max_seq_len = int(seq_lens[:num_decodes].max().item())
+        _C.pooled_window_attention_decode(
+            out, q, k_cache, v_cache, pool_k, pool_v, block_table,
+            query_start_loc, seq_lens, gate, scale, window, pool,
+            num_decodes, max_seq_len)
+        row0 = num_decodes
+    n_rows = (num_decodes if tiled else T) - row0
     if n_rows > 0:
         _C.pooled_window_attention_rows(
             out, q, k_cache, v_cache, pool_k, pool_v, block_table,
-            query_start_loc, seq_lens, gate, scale, window, pool, 0,
+            query_start_loc, seq_lens, gate, scale, window, pool, row0,
             n_rows)
     if tiled and num_decodes < num_reqs:
         if max_query_len <= 0:
