@@ -167,12 +167,15 @@ def test_far_key_on_gpu_bf16():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_elementwise_kernels(dtype):
+# Widths on the 4-wide kernels (one and several chunks per thread), an
+# odd width and one too wide for them (both on the scalar kernels).
+@pytest.mark.parametrize("W", [352, 2560, 355, 4100])
+def test_elementwise_kernels(dtype, W):
     from vllm_amd.ops import hip_ops as Hp
 
     torch.manual_seed(0)
     tol = 1e-5 if dtype == torch.float32 else 1e-2
-    W, T = 352, 37
+    T = 37
     y = _round(torch.randn(T, W), dtype)
     g = torch.tensor(0.7)
     _close(Hp.scalar_rms_norm(y.to("cuda", dtype), g.cuda(), 1e-5,
@@ -201,7 +204,11 @@ def test_elementwise_kernels(dtype):
         _close(sg[rows[r]], x[e - 1], 0)
     _close(sg[2], state[2], 0)
     # q/k head norm fused with the cache write
-    H, G, D, Dv, bs = 4, 2, 24, 40, 64
+    # 8-aligned head widths take the 16 B kernel (two chunks at 136);
+    # the others the scalar one.
+    H, G, D, Dv, bs = {352: (4, 2, 24, 40, 64), 2560: (5, 5, 136, 256, 64),
+                       355: (4, 2, 20, 40, 64),
+                       4100: (18, 1, 64, 8, 64)}[W]
     q = _round(torch.randn(T, H, D), dtype)
     k = _round(torch.randn(T, G, D), dtype)
     v = _round(torch.randn(T, G, Dv), dtype)

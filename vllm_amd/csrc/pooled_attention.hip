@@ -97,6 +97,66 @@ __global__ __launch_bounds__(EW_BLOCK) void add_scaled_scalar_norm_kernel(
   }
 }
 
+// 4-wide variants (width % 4 == 0, width <= 4 * EW_BLOCK * EW_VCH): 16 B
+// fp32 accesses, and the sublayer output stays in registers between the
+// sum of squares and the add.
+constexpr int EW_VCH = 4;
+
+template <typename T>
+DEVINL f32x4 ld4(const typename ET<T>::t* __restrict__ p) {
+  if constexpr (sizeof(typename ET<T>::t) == 4) {
+    return *reinterpret_cast<const f32x4*>(p);
+  } else {
+    const s16x4 v = *reinterpret_cast<const s16x4*>(p);
+    return f32x4{ET<T>::ld(v[0]), ET<T>::ld(v[1]), ET<T>::ld(v[2]),
+                 ET<T>::ld(v[3])};
+  }
+}
+
+template <typename T>
+DEVINL void st4(typename ET<T>::t* __restrict__ p, const f32x4 v) {
+  if constexpr (sizeof(typename ET<T>::t) == 4) {
+    *reinterpret_cast<f32x4*>(p) = v;
+  } else {
+    *reinterpret_cast<s16x4*>(p) =
+        s16x4{ET<T>::st(v[0]), ET<T>::st(v[1]), ET<T>::st(v[2]),
+              ET<T>::st(v[3])};
+  }
+}
+
+template <typename TY, typename TO>
+__global__ __launch_bounds__(EW_BLOCK) void add_scaled_scalar_norm_vec_kernel(
+    float* __restrict__ residual, const typename ET<TY>::t* __restrict__ y,
+    const float* __restrict__ gain, const float eps, const float mult,
+    const int width, typename ET<TO>::t* __restrict__ out_copy) {
+  __shared__ float scratch[4];
+  const int64_t row = blockIdx.x;
+  const typename ET<TY>::t* yr = y + row * width;
+  f32x4 yv[EW_VCH];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < EW_VCH; ++k) {
+    const int c = (k * EW_BLOCK + threadIdx.x) * 4;
+    yv[k] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < width) yv[k] = ld4<TY>(yr + c);
+    ss += yv[k][0] * yv[k][0] + yv[k][1] * yv[k][1] + yv[k][2] * yv[k][2] +
+          yv[k][3] * yv[k][3];
+  }
+  ss = block_sum_256(ss, scratch);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+  const float g = gain[0];
+#pragma unroll
+  for (int k = 0; k < EW_VCH; ++k) {
+    const int c = (k * EW_BLOCK + threadIdx.x) * 4;
+    if (c >= width) continue;
+    f32x4 r = *reinterpret_cast<const f32x4*>(residual + row * width + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = r[e] + mult * (yv[k][e] * inv * g);
+    *reinterpret_cast<f32x4*>(residual + row * width + c) = r;
+    if (out_copy != nullptr) st4<TO>(out_copy + row * width + c, r);
+  }
+}
+
 // Request that owns flat token t: largest r with qsl[r] <= t.
 DEVINL int find_req(const int* __restrict__ qsl, int num_reqs, int t) {
   int lo = 0, hi = num_reqs - 1;
@@ -124,6 +184,31 @@ __global__ __launch_bounds__(EW_BLOCK) void token_shift_kernel(
     const float h = xr[c];
     const float p = prev != nullptr ? prev[c] : 0.f;
     out[(int64_t)t * width + c] = ET<TO>::st(h + (p - h) * mu[c]);
+  }
+}
+
+template <typename TO>
+__global__ __launch_bounds__(EW_BLOCK) void token_shift_vec_kernel(
+    typename ET<TO>::t* __restrict__ out, const float* __restrict__ x,
+    const float* __restrict__ mu, const float* __restrict__ state,
+    const int64_t* __restrict__ state_rows, const int* __restrict__ qsl,
+    const int num_reqs, const int width) {
+  const int t = blockIdx.x;
+  const int r = find_req(qsl, num_reqs, t);
+  const bool first = (t == qsl[r]);
+  const float* prev = nullptr;
+  if (!first) prev = x + (int64_t)(t - 1) * width;
+  else if (state != nullptr) prev = state + state_rows[r] * width;
+  const float* xr = x + (int64_t)t * width;
+  for (int c = threadIdx.x * 4; c < width; c += EW_BLOCK * 4) {
+    const f32x4 h = *reinterpret_cast<const f32x4*>(xr + c);
+    const f32x4 m = *reinterpret_cast<const f32x4*>(mu + c);
+    f32x4 p = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (prev != nullptr) p = *reinterpret_cast<const f32x4*>(prev + c);
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = h[e] + (p[e] - h[e]) * m[e];
+    st4<TO>(out + (int64_t)t * width + c, o);
   }
 }
 
@@ -209,6 +294,79 @@ __global__ __launch_bounds__(EW_BLOCK) void norm_qk_cache_write_kernel(
     typename ET<T>::t* dst =
         v_cache + ((blk * G + head) * block_size + off) * Dv;
     for (int c = lane; c < Dv; c += 64) dst[c] = src[c];
+  }
+}
+
+// 16-bit, 8-aligned variant: 16 lanes per (token, head slot), 8 channels
+// = one 16 B access per lane and 128-channel stride; a 256-thread block
+// covers 16 head slots. Head widths up to 256 stay in registers.
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void norm_qk_cache_write_vec_kernel(
+    short* __restrict__ q_out, const short* __restrict__ q_in,
+    const int64_t q_stride, const short* __restrict__ k_in,
+    const int64_t k_stride, const short* __restrict__ v_in,
+    const int64_t v_stride, const short* __restrict__ q_w,
+    const short* __restrict__ k_w, const float eps,
+    short* __restrict__ k_cache, short* __restrict__ v_cache,
+    const int64_t* __restrict__ slot_mapping, const int H, const int G,
+    const int D, const int Dv, const int block_size) {
+  const int t = blockIdx.x;
+  const int slot_id = blockIdx.y * 16 + (threadIdx.x >> 4);
+  const int l16 = threadIdx.x & 15;
+  if (slot_id >= H + 2 * G) return;
+  const int64_t slot = slot_mapping[t];
+  const bool is_q = slot_id < H;
+  const bool is_v = slot_id >= H + G;
+  if (!is_q && slot < 0) return;
+  const int head = is_q ? slot_id : (is_v ? slot_id - H - G : slot_id - H);
+  const int W = is_v ? Dv : D;
+  const short* src = is_q ? q_in + t * q_stride + (int64_t)head * D
+                   : is_v ? v_in + t * v_stride + (int64_t)head * Dv
+                          : k_in + t * k_stride + (int64_t)head * D;
+  short* dst;
+  if (is_q) {
+    dst = q_out + ((int64_t)t * H + head) * D;
+  } else {
+    const int64_t blk = slot / block_size, off = slot % block_size;
+    dst = (is_v ? v_cache : k_cache) +
+          ((blk * G + head) * block_size + off) * W;
+  }
+  const short* w = is_q ? q_w : (is_v ? nullptr : k_w);
+  s16x8 raw[2];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int c = k * 128 + l16 * 8;
+    if (c < W) {
+      raw[k] = *reinterpret_cast<const s16x8*>(src + c);
+      if (w != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float f = ET<T>::ld(raw[k][e]);
+          ss += f * f;
+        }
+      }
+    }
+  }
+  if (w != nullptr) {
+    ss = group16_reduce_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int c = k * 128 + l16 * 8;
+      if (c < W) {
+        const s16x8 wv = *reinterpret_cast<const s16x8*>(w + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          raw[k][e] = ET<T>::st(ET<T>::ld(raw[k][e]) * inv *
+                                ET<T>::ld(wv[e]));
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int c = k * 128 + l16 * 8;
+    if (c < W) *reinterpret_cast<s16x8*>(dst + c) = raw[k];
   }
 }
 
@@ -408,7 +566,16 @@ torch::Tensor add_scaled_scalar_norm(torch::Tensor residual, torch::Tensor y,
                                residual.options().dtype(*out_dtype));
   if (rows == 0) return out;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool vec = width % 4 == 0 && width <= 4 * EW_BLOCK * EW_VCH;
 #define L2(TY, TO)                                                         \
+  if (vec)                                                                 \
+    hipLaunchKernelGGL((add_scaled_scalar_norm_vec_kernel<TY, TO>),        \
+                       dim3(rows), dim3(EW_BLOCK), 0, stream,              \
+                       residual.data_ptr<float>(),                         \
+                       (const ET<TY>::t*)y.data_ptr(),                     \
+                       gain.data_ptr<float>(), (float)eps, (float)mult,    \
+                       width, copy ? (ET<TO>::t*)out.data_ptr() : nullptr);\
+  else                                                                     \
   hipLaunchKernelGGL((add_scaled_scalar_norm_kernel<TY, TO>), dim3(rows),  \
                      dim3(EW_BLOCK), 0, stream, residual.data_ptr<float>(),\
                      (const ET<TY>::t*)y.data_ptr(), gain.data_ptr<float>(),\
@@ -449,7 +616,18 @@ torch::Tensor token_shift(torch::Tensor x, torch::Tensor mu,
                 state_rows->numel() >= num_reqs);
   }
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool vec = width % 4 == 0;
 #define L(TO)                                                              \
+  if (vec)                                                                 \
+    hipLaunchKernelGGL((token_shift_vec_kernel<TO>), dim3(T),              \
+                       dim3(EW_BLOCK), 0, stream,                          \
+                       (ET<TO>::t*)out.data_ptr(), x.data_ptr<float>(),    \
+                       mu.data_ptr<float>(),                               \
+                       has_state ? state->data_ptr<float>() : nullptr,     \
+                       has_state ? state_rows->data_ptr<int64_t>()         \
+                                 : nullptr,                                \
+                       query_start_loc.data_ptr<int>(), num_reqs, width);  \
+  else                                                                     \
   hipLaunchKernelGGL((token_shift_kernel<TO>), dim3(T), dim3(EW_BLOCK), 0, \
                      stream, (ET<TO>::t*)out.data_ptr(),                   \
                      x.data_ptr<float>(), mu.data_ptr<float>(),            \
@@ -524,6 +702,32 @@ torch::Tensor norm_qk_cache_write(torch::Tensor q, torch::Tensor k,
   auto q_out = torch::empty({T, H, D}, q.options());
   if (T == 0) return q_out;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  auto al16 = [](const torch::Tensor& x) {
+    return reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0;
+  };
+  const bool vec =
+      q.scalar_type() != torch::kFloat32 && D % 8 == 0 && Dv % 8 == 0 &&
+      D <= 256 && Dv <= 256 && q.stride(0) % 8 == 0 && k.stride(0) % 8 == 0 &&
+      v.stride(0) % 8 == 0 && al16(q) && al16(k) && al16(v) &&
+      (!q_w.has_value() || (al16(*q_w) && al16(*k_w)));
+  if (vec) {
+    dim3 vgrid(T, (H + 2 * G + 15) / 16);
+#define LV(TT)                                                             \
+  hipLaunchKernelGGL(                                                      \
+      (norm_qk_cache_write_vec_kernel<TT>), vgrid, dim3(EW_BLOCK), 0,      \
+      stream, (short*)q_out.data_ptr(), (const short*)q.data_ptr(),        \
+      q.stride(0), (const short*)k.data_ptr(), k.stride(0),                \
+      (const short*)v.data_ptr(), v.stride(0),                             \
+      q_w.has_value() ? (const short*)q_w->data_ptr() : nullptr,           \
+      k_w.has_value() ? (const short*)k_w->data_ptr() : nullptr,           \
+      (float)eps, (short*)k_cache.data_ptr(), (short*)v_cache.data_ptr(),  \
+      slot_mapping.data_ptr<int64_t>(), H, G, D, Dv, (int)k_cache.size(2))
+    if (q.scalar_type() == torch::kBFloat16) { LV(BF16Tag); }
+    else { LV(FP16Tag); }
+#undef LV
+    HIP_CHECK_KERNEL();
+    return q_out;
+  }
   dim3 grid(T, (H + 2 * G + 3) / 4);
 #define L(TT)                                                              \
   hipLaunchKernelGGL(                                                      \
