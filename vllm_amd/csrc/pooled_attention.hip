@@ -385,27 +385,27 @@ __global__ __launch_bounds__(EW_BLOCK) void pool_update_kernel(
   const int g = blockIdx.z;
   const int end = seq_lens[r];
   const int start = end - (qsl[r + 1] - qsl[r]);
-  const int b = start / P + blockIdx.y;
-  if (b >= end / P) return;
   const int* bt = block_table + (int64_t)r * max_blocks;
-  const int last = b * P + P - 1;
-  const int page = last / block_size;
-  const int slot = b - (page * block_size) / P;
-  const int64_t pb = bt[page];
   const float inv = 1.f / (float)P;
-  for (int c = threadIdx.x; c < D + Dv; c += EW_BLOCK) {
-    const bool is_k = c < D;
-    const int cc = is_k ? c : c - D;
-    const int W = is_k ? D : Dv;
-    const typename ET<T>::t* cache = is_k ? k_cache : v_cache;
-    float s = 0.f;
-    for (int p = b * P; p <= last; ++p) {
-      const int64_t blk = bt[p / block_size];
-      s += ET<T>::ld(
-          cache[((blk * G + g) * block_size + p % block_size) * W + cc]);
+  for (int b = start / P + blockIdx.y; b < end / P; b += gridDim.y) {
+    const int last = b * P + P - 1;
+    const int page = last / block_size;
+    const int slot = b - (page * block_size) / P;
+    const int64_t pb = bt[page];
+    for (int c = threadIdx.x; c < D + Dv; c += EW_BLOCK) {
+      const bool is_k = c < D;
+      const int cc = is_k ? c : c - D;
+      const int W = is_k ? D : Dv;
+      const typename ET<T>::t* cache = is_k ? k_cache : v_cache;
+      float s = 0.f;
+      for (int p = b * P; p <= last; ++p) {
+        const int64_t blk = bt[p / block_size];
+        s += ET<T>::ld(
+            cache[((blk * G + g) * block_size + p % block_size) * W + cc]);
+      }
+      float* dst = is_k ? pool_k : pool_v;
+      dst[((pb * G + g) * slots + slot) * W + cc] = s * inv;
     }
-    float* dst = is_k ? pool_k : pool_v;
-    dst[((pb * G + g) * slots + slot) * W + cc] = s * inv;
   }
 }
 
@@ -772,9 +772,12 @@ void pool_update(torch::Tensor k_cache, torch::Tensor v_cache,
               query_start_loc.size(0) >= num_reqs + 1);
   if (num_reqs == 0 || max_query_len <= 0) return;
   // A step of n tokens completes at most n / P + 1 pooled blocks.
+  // Workgroups stride over them, so a wide batch with one long chunk
+  // does not launch a grid of mostly idle workgroups.
   const int per_req = (int)(max_query_len / pool) + 1;
+  const int wide = std::max(1, 2048 / (num_reqs * G));
   auto stream = c10::hip::getCurrentHIPStream().stream();
-  dim3 grid(num_reqs, per_req, G);
+  dim3 grid(num_reqs, std::min(per_req, wide), G);
 #define L(TT)                                                              \
   hipLaunchKernelGGL((pool_update_kernel<TT>), grid, dim3(EW_BLOCK), 0,    \
                      stream, pool_k.data_ptr<float>(),                     \
