@@ -15,7 +15,7 @@ window, learned-router MoE) whose per-token active expert width matches
            context ~= prompt_len.
 
 One JSON line per (family, size, phase) goes to stdout. The default
-bench.py workload and its one-line contract are untouched.
+bench.py workload and its one-line output are untouched.
 """
 
 from __future__ import annotations

@@ -296,6 +296,30 @@ def test_engine_on_gpu(model_g, dtype, tol):
             _close(got[(r, p)], ref[p], tol)
 
 
+@pytest.mark.parametrize("dtype,tol", [("float32", 3e-4),
+                                       ("bfloat16", 0.15)])
+def test_unaligned_sizes_on_gpu(tmp_path, dtype, tol):
+    """Width, vocab, head and expert widths that are multiples of
+    neither 8 nor 16: the scalar kernels and the unaligned GEMM route."""
+    layers = [
+        O.layer_entry(heads=5, kv_heads=1, dim=24, vdim=40, window=9,
+                      pool=4, experts=5, top=2, ff=28, shared_ff=36),
+        O.layer_entry(heads=2, kv_heads=2, dim=20, vdim=12, window=33,
+                      pool=64, experts=2, top=2, ff=10, shared_ff=6),
+        O.layer_entry(heads=6, kv_heads=2, dim=8, vdim=8, window=64,
+                      pool=1, mlp=False),
+    ]
+    cfg = O.make_config(layers, vocab=101, width=100, residual_mult=0.7)
+    wt = O.random_weights(cfg, seed=9, sharp=2.0)
+    path = O.save_model(str(tmp_path / "m"), cfg, wt)
+    toks = _tokens(140, 101, 6)
+    ref = O.forward(cfg, wt, toks)
+    got, _ = run_schedule(path, chunked("a", toks, [3, 70, 2] + [1] * 65),
+                          dtype=dtype, device="cuda")
+    for p in range(len(toks)):
+        _close(got[("a", p)], ref[p], tol)
+
+
 def test_grouped_gemm_expert_path(tmp_path):
     """Widths that qualify for the grouped-GEMM MFMA expert kernels
     (width % 128 == 0, ff % 64 == 0, bf16)."""

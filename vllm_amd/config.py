@@ -1053,7 +1053,7 @@ def _gadilix_spec(path: str, cfg: dict) -> ModelSpec:
                 f"gadilix: layer {i} borrows weights of layer {j}, which "
                 "is not a layer with tensors of its own")
         mlp = entry.get("mlp")
-        if mlp is not None and mlp.get("kind") != "moe":
+        if mlp is not None and mlp.get("kind", "moe") != "moe":
             raise ValueError(
                 f"gadilix: layer {i} has unknown mlp kind "
                 f"{mlp.get('kind')!r}")

@@ -43,9 +43,9 @@ def apply_rope(positions, q, k, cos_sin_cache, rotary_dim, is_neox=True):
 
 
 def silu_and_mul(x):
-    if x.dtype == torch.float32:
-        # The 16-bit kernel above is vectorized for 2-byte elements;
-        # fp32 rows take the generic one.
+    if x.dtype == torch.float32 or (x.shape[-1] // 2) % 8:
+        # The 16-bit kernel is vectorized for 2-byte elements in groups
+        # of 8; fp32 rows and other widths take the generic one.
         shape = list(x.shape)
         out = _C.silu_and_mul_any(x.reshape(-1, shape[-1]).contiguous())
         shape[-1] //= 2

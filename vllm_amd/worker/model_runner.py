@@ -878,11 +878,13 @@ class ModelRunner:
             cur = self._row_pos[rows]
             self._row_pos[last_rows] = -1
             hit = cur >= 0
-            # Rows still inside their prompt feed the known prompt
-            # token, not a sampled one.
+            # Rows still inside their prompt (or replaying known
+            # tokens after a resume) feed the host-side token, not a
+            # sampled one.
             for j, r in enumerate(req_ids):
                 st = self.requests[r]
-                if st.num_computed_tokens < len(st.token_ids):
+                if (st.num_computed_tokens < st.prompt_len
+                        or st.num_computed_tokens + 1 < len(st.token_ids)):
                     hit[j] = False
             if hit.all():
                 idx = torch.from_numpy(cur).to(last_t.device)
