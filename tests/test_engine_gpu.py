@@ -205,7 +205,28 @@ def test_medusa_gpu_matches_baseline():
     sched = llm.engine.engine_core.scheduler
     assert sched.spec_stats_drafted > 0
     llm.shutdown()
-    assert base == med
+    if base == med:
+        return
+    # Verification steps run several rows per request through other
+    # GEMM shapes than one-row decode steps, so bf16 logits differ in
+    # their last bits and a near-tie of the random-weight model can
+    # flip. The first divergence must be such a tie in the baseline's
+    # own logits; anything else is a bookkeeping fault.
+    llm = _llm()
+    one = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True,
+                         logprobs=8)
+    try:
+        for prompt, a, b in zip(prompts, base, med):
+            if a == b:
+                continue
+            i = next(k for k, (x, y) in enumerate(zip(a, b)) if x != y)
+            out = llm.generate([prompt + list(a[:i])], one)
+            lp = out[0].outputs[0].logprobs[0]
+            assert a[i] in lp and b[i] in lp, (i, a, b, lp)
+            print("medusa tie:", i, a[i], b[i], lp[a[i]], lp[b[i]])
+            assert abs(lp[a[i]] - lp[b[i]]) < 0.03, (i, a, b, lp)
+    finally:
+        llm.shutdown()
 
 
 def test_sleep_wake_gpu():
