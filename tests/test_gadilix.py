@@ -161,6 +161,72 @@ def test_single_far_key_dominates():
             assert abs(out[i, 0, 0] - blk_mean) < 1e-3, (i, out[i, 0, 0])
 
 
+def test_output_gate_scales_each_head():
+    """The gate multiplies head h of token t by sigmoid(gate[t, h]); a
+    very negative gate silences one head and leaves the others."""
+    torch.manual_seed(4)
+    from vllm_amd import ops
+    T, H, G, D, Dv, Wn, P, bs = 70, 4, 2, 8, 6, 9, 4, 64
+    q, k, v = torch.randn(T, H, D), torch.randn(T, G, D), \
+        torch.randn(T, G, Dv)
+    gate = torch.randn(T, H)
+    gate[:, 2] = -40.0
+    ref = O.pooled_window_attention(q, k, v, 0.4, Wn, P) \
+        * torch.sigmoid(gate).unsqueeze(-1)
+    kc, vc = torch.zeros(3, G, bs, D), torch.zeros(3, G, bs, Dv)
+    slots = ops.pool_slots_per_page(P, bs)
+    pk, pv = torch.zeros(3, G, slots, D), torch.zeros(3, G, slots, Dv)
+    bt = torch.tensor([[2, 0, 1]], dtype=torch.int32)
+    pos = torch.arange(T)
+    slot = bt[0, pos // bs].long() * bs + pos % bs
+    qsl = torch.tensor([0, T], dtype=torch.int32)
+    sl = torch.tensor([T], dtype=torch.int32)
+    qq = ops.norm_qk_cache_write(q, k, v, None, None, 0.0, kc, vc, slot)
+    ops.pool_update(kc, vc, pk, pv, bt, qsl, sl, P, max_query_len=T)
+    out = ops.pooled_window_attention(qq, kc, vc, pk, pv, bt, qsl, sl, 0.4,
+                                      Wn, P, gate=gate, max_seq_len=T,
+                                      max_query_len=T)
+    _close(out, ref, 1e-5)
+    assert float(out[:, 2].abs().max()) < 1e-12
+
+
+def test_table_routed_experts_alone():
+    """The feed-forward module by itself: experts come from the token
+    id's table row with weight 1/top each, plus the shared expert; the
+    activations play no part in the choice."""
+    from vllm_amd.models.gadilix import GadilixMoE
+
+    torch.manual_seed(6)
+    V, W = 23, 16
+    for experts, top, shared in ((5, 2, 12), (3, 3, None), (4, 1, 8)):
+        ml = {"kind": "moe", "expert": {"ff": 10},
+              "router": {"experts": experts, "top": top}}
+        if shared:
+            ml["shared"] = {"ff": shared}
+        cfg = O.make_config([dict(O.layer_entry(), mlp=ml)], vocab=V,
+                            width=W)
+        wt = O.random_weights(cfg, seed=experts)
+        moe = GadilixMoE(W, V, ml, torch.float32)
+        moe.router.table.copy_(wt["l0.mlp.table"])
+        moe.experts.load_full_weights(
+            torch.stack([wt[f"l0.mlp.e{e}.gate"] for e in range(experts)]),
+            torch.stack([wt[f"l0.mlp.e{e}.up"] for e in range(experts)]),
+            torch.stack([wt[f"l0.mlp.e{e}.down"] for e in range(experts)]))
+        if shared:
+            moe.shared.gate_up_proj.weight.data.copy_(torch.cat(
+                [wt["l0.mlp.shared.gate"], wt["l0.mlp.shared.up"]]))
+            moe.shared.down_proj.weight.data.copy_(
+                wt["l0.mlp.shared.down"])
+        toks = torch.tensor([0, 22, 7, 7, 13, 1, 0])
+        x = torch.randn(len(toks), W)
+        want = O.table_moe(x, toks.tolist(), wt, "l0.mlp.", ml)
+        _close(moe(x, toks), want, 1e-5)
+        # Same token id, other activations: same experts.
+        x2 = torch.randn(len(toks), W) * 30
+        _close(moe(x2, toks), O.table_moe(x2, toks.tolist(), wt,
+                                          "l0.mlp.", ml), 1e-4)
+
+
 # ---------------------------------------------------------------------
 # The engine against whole-sequence oracle logits.
 
