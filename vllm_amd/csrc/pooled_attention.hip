@@ -124,6 +124,38 @@ DEVINL void st4(typename ET<T>::t* __restrict__ p, const f32x4 v) {
   }
 }
 
+template <typename TI, typename TO>
+__global__ __launch_bounds__(EW_BLOCK) void scalar_rms_norm_vec_kernel(
+    typename ET<TO>::t* __restrict__ out,
+    const typename ET<TI>::t* __restrict__ x, const float* __restrict__ gain,
+    const float eps, const int width) {
+  __shared__ float scratch[4];
+  const int64_t row = blockIdx.x;
+  const typename ET<TI>::t* xr = x + row * width;
+  f32x4 xv[EW_VCH];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < EW_VCH; ++k) {
+    const int c = (k * EW_BLOCK + threadIdx.x) * 4;
+    xv[k] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < width) xv[k] = ld4<TI>(xr + c);
+    ss += xv[k][0] * xv[k][0] + xv[k][1] * xv[k][1] + xv[k][2] * xv[k][2] +
+          xv[k][3] * xv[k][3];
+  }
+  ss = block_sum_256(ss, scratch);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+  const float g = gain[0];
+#pragma unroll
+  for (int k = 0; k < EW_VCH; ++k) {
+    const int c = (k * EW_BLOCK + threadIdx.x) * 4;
+    if (c >= width) continue;
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = xv[k][e] * inv * g;
+    st4<TO>(out + row * width + c, o);
+  }
+}
+
 template <typename TY, typename TO>
 __global__ __launch_bounds__(EW_BLOCK) void add_scaled_scalar_norm_vec_kernel(
     float* __restrict__ residual, const typename ET<TY>::t* __restrict__ y,
@@ -398,6 +430,7 @@ __global__ __launch_bounds__(EW_BLOCK) void pool_update_kernel(
       const int W = is_k ? D : Dv;
       const typename ET<T>::t* cache = is_k ? k_cache : v_cache;
       float s = 0.f;
+#pragma unroll 4
       for (int p = b * P; p <= last; ++p) {
         const int64_t blk = bt[p / block_size];
         s += ET<T>::ld(
@@ -406,6 +439,70 @@ __global__ __launch_bounds__(EW_BLOCK) void pool_update_kernel(
       float* dst = is_k ? pool_k : pool_v;
       dst[((pb * G + g) * slots + slot) * W + cc] = s * inv;
     }
+  }
+}
+
+// 16-bit, 8-aligned variant: (D + Dv) / 8 lanes cover one position with
+// 16 B loads and the remaining threads take other positions of the
+// block, so a block of P positions costs P * (D + Dv) / 2048 dependent
+// loads per thread instead of P. Position slices merge through LDS in a
+// fixed order (the mean of a block never depends on the step that
+// finished it).
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void pool_update_vec_kernel(
+    float* __restrict__ pool_k, float* __restrict__ pool_v,
+    const short* __restrict__ k_cache, const short* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int max_blocks,
+    const int* __restrict__ qsl, const int* __restrict__ seq_lens,
+    const int G, const int D, const int Dv, const int block_size,
+    const int P, const int slots) {
+  __shared__ float red[EW_BLOCK][9];     // padded: no bank conflicts
+  const int r = blockIdx.x;
+  const int g = blockIdx.z;
+  const int end = seq_lens[r];
+  const int start = end - (qsl[r + 1] - qsl[r]);
+  const int* bt = block_table + (int64_t)r * max_blocks;
+  const float inv = 1.f / (float)P;
+  const int LP = (D + Dv) / 8;           // lanes per position
+  const int NS = EW_BLOCK / LP;          // position slices
+  const int lane = threadIdx.x % LP;
+  const int slice = threadIdx.x / LP;
+  const bool is_k = lane * 8 < D;
+  const int cc = is_k ? lane * 8 : lane * 8 - D;
+  const int W = is_k ? D : Dv;
+  const short* cache = is_k ? k_cache : v_cache;
+  for (int b = start / P + blockIdx.y; b < end / P; b += gridDim.y) {
+    const int last = b * P + P - 1;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    if (slice < NS) {
+#pragma unroll 4
+      for (int p = b * P + slice; p <= last; p += NS) {
+        const int64_t blk = bt[p / block_size];
+        const s16x8 v = *reinterpret_cast<const s16x8*>(
+            cache + ((blk * G + g) * block_size + p % block_size) * W + cc);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += ET<T>::ld(v[e]);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[threadIdx.x][e] = acc[e];
+    __syncthreads();
+    if (slice == 0) {
+      const int page = last / block_size;
+      const int slot = b - (page * block_size) / P;
+      const int64_t pb = bt[page];
+      float* dst = (is_k ? pool_k : pool_v) +
+                   ((pb * G + g) * slots + slot) * W + cc;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float t = 0.f;
+        for (int sl = 0; sl < NS; ++sl) t += red[sl * LP + lane][e];
+        dst[e] = t * inv;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -533,7 +630,15 @@ torch::Tensor scalar_rms_norm(torch::Tensor x, torch::Tensor gain,
   const int rows = x.size(0), width = x.size(1);
   if (rows == 0) return out;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool vec = width % 4 == 0 && width <= 4 * EW_BLOCK * EW_VCH;
 #define L2(TI, TO)                                                         \
+  if (vec)                                                                 \
+    hipLaunchKernelGGL((scalar_rms_norm_vec_kernel<TI, TO>), dim3(rows),   \
+                       dim3(EW_BLOCK), 0, stream,                          \
+                       (ET<TO>::t*)out.data_ptr(),                         \
+                       (const ET<TI>::t*)x.data_ptr(),                     \
+                       gain.data_ptr<float>(), (float)eps, width);         \
+  else                                                                     \
   hipLaunchKernelGGL((scalar_rms_norm_kernel<TI, TO>), dim3(rows),         \
                      dim3(EW_BLOCK), 0, stream,                            \
                      (ET<TO>::t*)out.data_ptr(),                           \
@@ -775,9 +880,27 @@ void pool_update(torch::Tensor k_cache, torch::Tensor v_cache,
   // Workgroups stride over them, so a wide batch with one long chunk
   // does not launch a grid of mostly idle workgroups.
   const int per_req = (int)(max_query_len / pool) + 1;
-  const int wide = std::max(1, 2048 / (num_reqs * G));
+  const int wide = std::max(1, 8192 / (num_reqs * G));
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid(num_reqs, std::min(per_req, wide), G);
+  if (k_cache.scalar_type() != torch::kFloat32 && D % 8 == 0 &&
+      Dv % 8 == 0 && (D + Dv) / 8 <= EW_BLOCK) {
+#define LV(TT)                                                             \
+  hipLaunchKernelGGL((pool_update_vec_kernel<TT>), grid, dim3(EW_BLOCK), 0,\
+                     stream, pool_k.data_ptr<float>(),                     \
+                     pool_v.data_ptr<float>(),                             \
+                     (const short*)k_cache.data_ptr(),                     \
+                     (const short*)v_cache.data_ptr(),                     \
+                     block_table.data_ptr<int>(), (int)block_table.size(1),\
+                     query_start_loc.data_ptr<int>(),                      \
+                     seq_lens.data_ptr<int>(), G, D, Dv, bs, (int)pool,    \
+                     slots)
+    if (k_cache.scalar_type() == torch::kBFloat16) { LV(BF16Tag); }
+    else { LV(FP16Tag); }
+#undef LV
+    HIP_CHECK_KERNEL();
+    return;
+  }
 #define L(TT)                                                              \
   hipLaunchKernelGGL((pool_update_kernel<TT>), grid, dim3(EW_BLOCK), 0,    \
                      stream, pool_k.data_ptr<float>(),                     \
