@@ -13,7 +13,7 @@ import torch
 
 
 def run_schedule(model_dir, steps, dtype="float32", max_tokens=1024,
-                 device="cpu"):
+                 device="cpu", enforce_eager=True):
     """steps: list of (entries, end) with entries = [(req_id, tokens,
     want_offsets)]. Returns {(req_id, absolute position): logits}."""
     from vllm_amd.entrypoints.trace_replay import build_core, replay
@@ -34,7 +34,8 @@ def run_schedule(model_dir, steps, dtype="float32", max_tokens=1024,
                                  "end": list(end)}))
         wanted.append(row)
     out = tempfile.mkdtemp()
-    core = build_core(model_dir, dtype, max_tokens, device)
+    core = build_core(model_dir, dtype, max_tokens, device,
+                      enforce_eager=enforce_eager)
     done = []
     try:
         replay(core, lines, out, done.append)

@@ -337,6 +337,49 @@ def test_grouped_gemm_expert_path(tmp_path):
         _close(got[("a", p)], ref[p], 0.15)
 
 
+def test_captured_decode_matches_eager(tmp_path):
+    """One-token steps replayed from captured hipGraphs (batch buckets
+    with padded rows, requests joining and leaving, state rows staged
+    per step) against the eager engine and the oracle."""
+    layers = [O.layer_entry(heads=4, kv_heads=2, dim=64, vdim=32,
+                            window=30, pool=8, experts=6, top=2, ff=64,
+                            shared_ff=128),
+              O.layer_entry(heads=4, kv_heads=2, dim=64, vdim=32,
+                            window=30, pool=8, experts=6, top=2, ff=64,
+                            shared_ff=128, weights_of=0),
+              O.layer_entry(heads=8, kv_heads=1, dim=32, vdim=64,
+                            window=300, pool=5, mlp=False)]
+    cfg = O.make_config(layers, vocab=80, width=256, residual_mult=0.35)
+    wt = O.random_weights(cfg, seed=5, sharp=2.0)
+    path = O.save_model(str(tmp_path / "m"), cfg, wt)
+    reqs = {"a": _tokens(150, 80, 41), "b": _tokens(90, 80, 42),
+            "c": _tokens(70, 80, 43)}
+    steps = [([("a", reqs["a"][:100], [99]), ("b", reqs["b"][:50], [49])],
+              [])]
+    for i in range(40):                       # two decode rows
+        steps.append(([("a", reqs["a"][100 + i:101 + i], [0]),
+                       ("b", reqs["b"][50 + i:51 + i], [0])],
+                      ["b"] if i == 39 else []))
+    steps.append(([("c", reqs["c"][:60], [59])], []))
+    for i in range(10):                       # other rows, other bucket
+        steps.append(([("a", reqs["a"][140 + i:141 + i], [0]),
+                       ("c", reqs["c"][60 + i:61 + i], [0])],
+                      ["a", "c"] if i == 9 else []))
+    graph, core = run_schedule(path, steps, dtype="bfloat16",
+                               device="cuda", enforce_eager=False)
+    assert core.worker.runner.graph_runner is not None
+    assert core.worker.runner.graph_runner.graphs, "nothing was captured"
+    eager, _ = run_schedule(path, steps, dtype="bfloat16", device="cuda")
+    assert graph.keys() == eager.keys()
+    for r, t in reqs.items():
+        ref = O.forward(cfg, wt, t)
+        for (rid, p_), got in graph.items():
+            if rid != r:
+                continue
+            _close(got, eager[(rid, p_)], 2e-2)
+            _close(got, ref[p_], 0.15)
+
+
 def test_greedy_generation_on_gpu(model_g):
     from vllm_amd.entrypoints.llm import LLM
     from vllm_amd.sampling_params import SamplingParams

@@ -126,6 +126,13 @@ __global__ __launch_bounds__(PD_BLOCK) void pwa_decode_kernel(
   pd_key_range(i, window, P, lo, nb, n_keys);
   const int j_begin = part * PD_PART;
   const int j_end = min(n_keys, j_begin + PD_PART);
+  if (n_keys <= 0) {
+    // Inert row (a padded entry of a captured batch): defined output.
+    if (part == 0)
+      for (int idx = threadIdx.x; idx < nh * Dv; idx += PD_BLOCK)
+        out[((int64_t)t * H + h0 + idx / Dv) * Dv + idx % Dv] = 0;
+    return;
+  }
   if (j_begin >= j_end) return;
 
   const int slot = threadIdx.x / LPT;
@@ -248,6 +255,7 @@ __global__ __launch_bounds__(PD_BLOCK) void pwa_decode_merge_kernel(
   int lo, nb, n_keys;
   pd_key_range(seq_lens[r] - 1, window, P, lo, nb, n_keys);
   const int used = min(n_parts, (n_keys + PD_PART - 1) / PD_PART);
+  if (used <= 0) return;                 // inert row: zeros already written
   const int64_t p0 = ((int64_t)r * H + h) * n_parts;
   float M = PD_NEG;
   for (int p = 0; p < used; ++p) M = fmaxf(M, tmp_ml[(p0 + p) * 2]);

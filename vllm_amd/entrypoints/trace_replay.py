@@ -37,7 +37,7 @@ MAX_LIVE_REQUESTS = 4
 
 
 def build_core(model_dir: str, dtype: str, max_tokens: int,
-               device: str = "auto"):
+               device: str = "auto", enforce_eager: bool = True):
     from vllm_amd.engine.arg_utils import EngineArgs
     from vllm_amd.engine.core import EngineCore
 
@@ -55,7 +55,9 @@ def build_core(model_dir: str, dtype: str, max_tokens: int,
         max_num_batched_tokens=num_blocks * block_size,
         enable_prefix_caching=False,
         async_scheduling=False,
-        enforce_eager=True,
+        # Eager by default: a replay is short and its batch shapes
+        # change every step, so captures would not pay for themselves.
+        enforce_eager=enforce_eager,
         device=device,
     )
     return EngineCore(args.create_engine_config())

@@ -127,8 +127,15 @@ class DecodeGraphRunner:
                                              dtype=torch.int32, device=dev)
             self.pin_bt_w = torch.empty(n, self.max_blocks,
                                         dtype=torch.int32, pin_memory=True)
+        # Row-state models (token-shift carry): the state row of each
+        # batch entry; padded entries point at the scratch row.
+        self.row_state = runner.spec.has_token_shift
+        self.scratch_row = cfg.scheduler_config.max_num_seqs
+        if self.row_state:
+            self.state_rows = torch.full((n,), self.scratch_row,
+                                         dtype=torch.int64, device=dev)
         # Pinned staging buffers for async H2D.
-        self.pin_i64 = torch.empty(4, n, dtype=torch.int64, pin_memory=True)
+        self.pin_i64 = torch.empty(5, n, dtype=torch.int64, pin_memory=True)
         self.pin_seq = torch.empty(n, dtype=torch.int32, pin_memory=True)
         self.pin_bt = torch.empty(n, self.max_blocks, dtype=torch.int32,
                                   pin_memory=True)
@@ -163,13 +170,18 @@ class DecodeGraphRunner:
                            if self.mixed_attn else None),
             slot_mapping_w=(self.slot_mapping_w[:nb]
                             if self.mixed_attn else None),
+            state_rows=(self.state_rows[:nb] if self.row_state else None),
         )
 
     def _capture(self, nb: int, parts: int):
         runner = self.runner
         ctx = ForwardContext(attn_metadata=self._meta(nb, parts),
                              kv_caches=runner.kv_caches,
-                             sp_size=self.sp_size)
+                             sp_size=self.sp_size,
+                             shift_states=runner.shift_states)
+        if self.row_state:
+            # The warmup pass below must not touch a live request's row.
+            self.state_rows[:nb].fill_(self.scratch_row)
         # Warmup on a side stream (allocator state, RCCL lazy init).
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -190,7 +202,8 @@ class DecodeGraphRunner:
     def run(self, n: int, nb: int, parts: int, input_ids, positions,
             slot_mapping, seq_lens, block_table,
             ids_dev: Optional[torch.Tensor] = None,
-            slot_mapping_w=None, block_table_w=None) -> torch.Tensor:
+            slot_mapping_w=None, block_table_w=None,
+            state_rows=None) -> torch.Tensor:
         """Stage inputs (n real rows, nb bucket) and replay. Returns
         logits for the n real rows. ids_dev, when given, is a device
         tensor of decode input ids (previous step's sampled tokens — no
@@ -224,6 +237,11 @@ class DecodeGraphRunner:
         entry = self.graphs.get((nb, parts))
         if entry is None:
             entry = self._capture(nb, parts)
+        if self.row_state:
+            # After a capture (its warmup ran on the scratch row).
+            pi[4, :n] = torch.from_numpy(state_rows)
+            pi[4, n:nb] = self.scratch_row
+            self.state_rows[:nb].copy_(pi[4, :nb], non_blocking=True)
         graph, logits, hidden = entry
         graph.replay()
         self.last_hidden = hidden
@@ -502,9 +520,18 @@ class ModelRunner:
                     torch.zeros(num_blocks, g, slots, dv,
                                 dtype=torch.float32, device=self.device),
                 ))
-            # Decode stays eager: state rows are dynamic indices and the
-            # expert path may synchronize with the host.
+            # Decode is captured when every layer's experts qualify for
+            # the grouped-GEMM kernels (no host sync) in a 16-bit dtype;
+            # state rows are staged into a static index buffer.
             self.graph_runner = None
+            if (self.device.type == "cuda"
+                    and not self.config.model_config.enforce_eager
+                    and not self.config.model_config.lora_modules
+                    and self.pp_size == 1 and get_tp_world_size() == 1
+                    and self.dtype in (torch.bfloat16, torch.float16)
+                    and all(self._experts_capturable(e)
+                            for e in spec.layer_specs)):
+                self.graph_runner = DecodeGraphRunner(self)
             return
         if spec.has_mamba:
             # SSM state: constant-size recurrent state per request row
@@ -588,6 +615,15 @@ class ModelRunner:
                 and self.pp_size == 1
                 and tp_graph_ok and moe_graph_ok and mla_graph_ok):
             self.graph_runner = DecodeGraphRunner(self)
+
+    def _experts_capturable(self, entry: dict) -> bool:
+        """Shapes of one layer's routed experts fit the grouped-GEMM
+        kernels (width % 128, ff % 64), or the layer has none."""
+        ml = entry.get("mlp")
+        if ml is None:
+            return True
+        ff = int(ml["expert"]["ff"])
+        return self.spec.hidden_size % 128 == 0 and ff % 64 == 0
 
     def allocate_host_kv_pool(self, num_host_blocks: int) -> None:
         """Pinned host-RAM pool for offloaded prefix blocks: one tensor
@@ -923,6 +959,8 @@ class ModelRunner:
                     seq_lens, block_table, ids_dev=ids_dev,
                     slot_mapping_w=slot_mapping_w,
                     block_table_w=block_table_w,
+                    state_rows=(rows.astype(np.int64)
+                                if self.has_row_state else None),
                 )
                 hidden = self.graph_runner.last_hidden
             except Exception:  # noqa: BLE001
