@@ -52,7 +52,7 @@ def _gadilix_dir(s: dict) -> str:
                 "shared": {"ff": s["ff"]}},
     }
     cfg = {"architecture": "Gadilix", "vocab": s["vocab"],
-           "width": s["width"], "residual_mult": 0.3,
+           "width": s["width"], "residual_mult": 0.5,
            "norm": {"eps": 1e-5}, "layers": [layer] * s["layers"]}
     d = tempfile.mkdtemp(prefix="gadilix_bench_")
     with open(os.path.join(d, "config.json"), "w") as f:
