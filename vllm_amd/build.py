@@ -31,6 +31,9 @@ SOURCES = [
     CSRC / "pooled_attention.hip",
     CSRC / "pooled_attention_prefill.hip",
     CSRC / "pooled_attention_decode.hip",
+    CSRC / "residual_ops.hip",
+    CSRC / "latent_attention.hip",
+    CSRC / "ssd.hip",
     CSRC / "gemm_hipblaslt.cpp",
     CSRC / "bindings.cpp",
 ]

@@ -119,6 +119,10 @@ class ModelSpec:
     layer_specs: Optional[list] = None
     # Multiplier on every sublayer's contribution to the residual sum.
     residual_mult: float = 1.0
+    # Multiplier on the token embedding (architecture "papunex").
+    embedding_scale: float = 1.0
+    # logits <- cap * tanh(logits / cap); 0 = off.
+    logit_softcap: float = 0.0
 
     @property
     def has_token_shift(self) -> bool:
@@ -132,7 +136,16 @@ class ModelSpec:
         paged blocks (SSM state, token-shift carry). Such state is not
         content-addressable, so prefix caching is off for these models
         and rows are cleared on (re)admission."""
-        return self.has_mamba or self.has_token_shift
+        return (self.has_mamba or self.has_token_shift
+                or self.has_layer_state)
+
+    @property
+    def has_layer_state(self) -> bool:
+        """Layer-listed stacks whose recurrent layers keep their state
+        in runner rows, one (conv tail, recurrent state) pair per such
+        layer (architecture "papunex", mixer type "mamba2")."""
+        return (self.architecture == "papunex"
+                and any(e["type"] == "mamba2" for e in self.layer_specs))
 
     @property
     def is_moe(self) -> bool:
@@ -1078,6 +1091,78 @@ def _gadilix_spec(path: str, cfg: dict) -> ModelSpec:
     )
 
 
+def _papunex_spec(path: str, cfg: dict) -> ModelSpec:
+    """Papunex config.json: {"architecture", "vocab", "width",
+    "embedding": {"scale"}, "norm": {"eps"}, "logit_softcap",
+    "layers": [{"type": "latent_attention" | "mamba2", "mixer": {...},
+    "mlp": {"kind": "dense" | "moe", ...} | null}]}. Sizes and constants
+    are per layer; the flat attention fields only give generic sizing
+    code something sane to read."""
+    layers = cfg["layers"]
+    if not layers:
+        raise ValueError("papunex: config lists no layers")
+    for i, entry in enumerate(layers):
+        kind, mx = entry.get("type"), entry.get("mixer") or {}
+        if kind == "latent_attention":
+            j = mx.get("kv_from")
+            if j is not None:
+                src = layers[j] if 0 <= j < i else None
+                smx = (src or {}).get("mixer") or {}
+                if (src is None or src.get("type") != "latent_attention"
+                        or smx.get("kv_from") is not None):
+                    raise ValueError(
+                        f"papunex: layer {i} reads the keys of layer {j}, "
+                        "which is not an earlier latent-attention layer "
+                        "with a key projection of its own")
+                if any(smx.get(k) != mx.get(k)
+                       for k in ("kv_rank", "rot_dim", "rot")):
+                    raise ValueError(
+                        f"papunex: layers {i} and {j} share keys but "
+                        "differ in kv_rank, rot_dim or rotation")
+            rot = mx.get("rot") or {}
+            if int(rot.get("dims", 0)) % 2 or not (
+                    0 <= int(rot.get("dims", 0)) <= int(mx["rot_dim"])):
+                raise ValueError(
+                    f"papunex: layer {i}: rot.dims must be even and at "
+                    "most rot_dim")
+        elif kind == "mamba2":
+            if (mx["heads"] % mx["groups"]
+                    or (mx["heads"] * mx["vdim"]) % mx["norm_groups"]):
+                raise ValueError(
+                    f"papunex: layer {i}: heads must divide into groups "
+                    "and the inner width into norm_groups")
+        else:
+            raise ValueError(
+                f"papunex: layer {i} has unknown mixer type {kind!r}")
+        mlp = entry.get("mlp")
+        if mlp is not None and mlp.get("kind") not in ("dense", "moe"):
+            raise ValueError(
+                f"papunex: layer {i} has unknown mlp kind "
+                f"{mlp.get('kind')!r}")
+    att = [e["mixer"] for e in layers if e["type"] == "latent_attention"]
+    return ModelSpec(
+        name=os.path.basename(path.rstrip("/")) or "papunex",
+        architecture="papunex",
+        vocab_size=cfg["vocab"],
+        hidden_size=cfg["width"],
+        intermediate_size=0,
+        num_layers=len(layers),
+        num_heads=max([m["heads"] for m in att] or [1]),
+        num_kv_heads=1,
+        head_dim=max([m["dim"] + m["rot_dim"] for m in att] or [1]),
+        rms_norm_eps=cfg["norm"]["eps"],
+        # Rotation angles are computed from the position itself; no
+        # table bounds the context.
+        max_position_embeddings=1 << 24,
+        layer_specs=layers,
+        embedding_scale=float((cfg.get("embedding") or {}).get("scale",
+                                                               1.0)),
+        logit_softcap=float(cfg.get("logit_softcap") or 0.0),
+        eos_token_id=-1,
+        bos_token_id=0,
+    )
+
+
 def _spec_from_hf_config(path: str) -> ModelSpec:
     """Build a ModelSpec from a local HF config.json directory/file."""
     cfg_path = path if path.endswith(".json") else os.path.join(path, "config.json")
@@ -1085,6 +1170,8 @@ def _spec_from_hf_config(path: str) -> ModelSpec:
         hf = json.load(f)
     if str(hf.get("architecture", "")).lower() == "gadilix":
         return _gadilix_spec(path, hf)
+    if str(hf.get("architecture", "")).lower() == "papunex":
+        return _papunex_spec(path, hf)
     arch = (hf.get("architectures") or ["LlamaForCausalLM"])[0].lower()
     if "jamba" in arch:
         # HF JambaForCausalLM: hybrid attn/mamba layer pattern + SSM

@@ -95,6 +95,46 @@ void pooled_window_attention_decode(
     torch::Tensor block_table, torch::Tensor query_start_loc,
     torch::Tensor seq_lens, c10::optional<torch::Tensor> gate, double scale,
     int64_t window, int64_t pool, int64_t num_decodes, int64_t max_seq_len);
+torch::Tensor scaled_embedding(torch::Tensor ids, torch::Tensor table,
+                               double scale);
+torch::Tensor rms_norm_cast(torch::Tensor x, torch::Tensor weight,
+                            double eps, torch::ScalarType out_dtype);
+torch::Tensor add_rms_norm(torch::Tensor residual, torch::Tensor y,
+                           torch::Tensor weight, double eps,
+                           c10::optional<torch::ScalarType> out_dtype);
+torch::Tensor relu2(torch::Tensor x);
+torch::Tensor logit_softcap(torch::Tensor logits, double cap);
+torch::Tensor sigmoid_gate_mul(torch::Tensor x, torch::Tensor gate);
+void latent_rope_cache_write(torch::Tensor q,
+                             c10::optional<torch::Tensor> dkv,
+                             c10::optional<torch::Tensor> norm_w, double eps,
+                             torch::Tensor positions, torch::Tensor inv_freq,
+                             int64_t nope_dim, int64_t kv_rank,
+                             c10::optional<torch::Tensor> cache,
+                             c10::optional<torch::Tensor> slot_mapping);
+void latent_attention_rows(torch::Tensor out, torch::Tensor q_abs,
+                           torch::Tensor q_rot, torch::Tensor cache,
+                           torch::Tensor block_table,
+                           torch::Tensor query_start_loc,
+                           torch::Tensor seq_lens,
+                           c10::optional<torch::Tensor> sink, double scale);
+torch::Tensor causal_conv_silu(torch::Tensor x, torch::Tensor weight,
+                               torch::Tensor bias,
+                               c10::optional<torch::Tensor> conv_state,
+                               c10::optional<torch::Tensor> state_rows,
+                               torch::Tensor query_start_loc,
+                               torch::ScalarType out_dtype);
+torch::Tensor ssd_scan(torch::Tensor xbc, int64_t heads, int64_t head_dim,
+                       int64_t groups, int64_t state, torch::Tensor dt,
+                       torch::Tensor dt_bias, torch::Tensor a_log,
+                       torch::Tensor d_skip,
+                       c10::optional<torch::Tensor> ssm_state,
+                       c10::optional<torch::Tensor> state_rows,
+                       torch::Tensor query_start_loc);
+torch::Tensor gated_group_rms_norm(torch::Tensor y, torch::Tensor z,
+                                   torch::Tensor weight, double eps,
+                                   int64_t groups,
+                                   torch::ScalarType out_dtype);
 torch::Tensor car_init(int64_t rank, int64_t world, int64_t max_bytes);
 void car_connect(torch::Tensor handles);
 bool car_is_ready();
@@ -173,6 +213,29 @@ TORCH_LIBRARY(vllm_amd, m) {
         "Tensor block_table, Tensor query_start_loc, Tensor seq_lens, "
         "Tensor? gate, float scale, int window, int pool, int num_decodes, "
         "int max_seq_len) -> ()");
+  m.def("scaled_embedding(Tensor ids, Tensor table, float scale) -> Tensor");
+  m.def("rms_norm_cast(Tensor x, Tensor weight, float eps, "
+        "ScalarType out_dtype) -> Tensor");
+  m.def("add_rms_norm(Tensor(a!) residual, Tensor y, Tensor weight, "
+        "float eps, ScalarType? out_dtype) -> Tensor");
+  m.def("relu2(Tensor x) -> Tensor");
+  m.def("logit_softcap(Tensor logits, float cap) -> Tensor");
+  m.def("sigmoid_gate_mul(Tensor x, Tensor gate) -> Tensor");
+  m.def("latent_rope_cache_write(Tensor(a!) q, Tensor? dkv, Tensor? norm_w, "
+        "float eps, Tensor positions, Tensor inv_freq, int nope_dim, "
+        "int kv_rank, Tensor(b!)? cache, Tensor? slot_mapping) -> ()");
+  m.def("latent_attention_rows(Tensor(a!) out, Tensor q_abs, Tensor q_rot, "
+        "Tensor cache, Tensor block_table, Tensor query_start_loc, "
+        "Tensor seq_lens, Tensor? sink, float scale) -> ()");
+  m.def("causal_conv_silu(Tensor x, Tensor weight, Tensor bias, "
+        "Tensor(a!)? conv_state, Tensor? state_rows, "
+        "Tensor query_start_loc, ScalarType out_dtype) -> Tensor");
+  m.def("ssd_scan(Tensor xbc, int heads, int head_dim, int groups, "
+        "int state, Tensor dt, Tensor dt_bias, Tensor a_log, "
+        "Tensor d_skip, Tensor(a!)? ssm_state, Tensor? state_rows, "
+        "Tensor query_start_loc) -> Tensor");
+  m.def("gated_group_rms_norm(Tensor y, Tensor z, Tensor weight, "
+        "float eps, int groups, ScalarType out_dtype) -> Tensor");
   // Custom xGMI collectives (comms.hip). init/connect/destroy are
   // host-side control ops and live on the catch-all dispatch below.
   m.def("car_init(int rank, int world, int max_bytes) -> Tensor");
@@ -225,4 +288,15 @@ TORCH_LIBRARY_IMPL(vllm_amd, CUDA, m) {
          &vllm_amd::pooled_window_attention_rows);
   m.impl("pooled_window_attention_decode",
          &vllm_amd::pooled_window_attention_decode);
+  m.impl("scaled_embedding", &vllm_amd::scaled_embedding);
+  m.impl("rms_norm_cast", &vllm_amd::rms_norm_cast);
+  m.impl("add_rms_norm", &vllm_amd::add_rms_norm);
+  m.impl("relu2", &vllm_amd::relu2);
+  m.impl("logit_softcap", &vllm_amd::logit_softcap);
+  m.impl("sigmoid_gate_mul", &vllm_amd::sigmoid_gate_mul);
+  m.impl("latent_rope_cache_write", &vllm_amd::latent_rope_cache_write);
+  m.impl("latent_attention_rows", &vllm_amd::latent_attention_rows);
+  m.impl("causal_conv_silu", &vllm_amd::causal_conv_silu);
+  m.impl("ssd_scan", &vllm_amd::ssd_scan);
+  m.impl("gated_group_rms_norm", &vllm_amd::gated_group_rms_norm);
 }

@@ -176,7 +176,7 @@ class EngineArgs:
             # pooler needs: encoders run whole-prompt, uncached.
             enable_prefix_caching = False
             enable_chunked_prefill = False
-        if spec.has_mamba:
+        if spec.has_mamba or spec.has_layer_state:
             # SSM state is not content-addressable: a prefix hit would
             # skip tokens the recurrent state never saw. Every
             # (re)admission scans from position 0.

@@ -168,3 +168,74 @@ class PooledWindowAttention(nn.Module):
             out = out * torch.sigmoid(gate.float()).unsqueeze(-1).to(
                 out.dtype)
         return out.reshape(q.shape[0], -1)
+
+
+class LatentAttention(nn.Module):
+    """Attention whose keys and values are both read from one cached
+    latent row per token, shared by all heads: cache row = [c (kv_rank)
+    | kr (rot_dim)]. A head's unrotated key is W_uk c and its value
+    W_uv c, so the layer never expands them: queries are carried into
+    the latent space (q_abs = W_uk^T q_nope, done by the caller), scores
+    are (q_abs . c + q_rot . kr) * scale, and the kernel returns the
+    attention-weighted latent [T, H, kv_rank] for the caller to expand
+    through W_uv. Causal over the whole context.
+
+    `sink` (one fp32 number per head, optional) is added to the softmax
+    denominator as exp(sink_h): it has no key and no value.
+
+    The same fused pass that writes the cache normalises c (RMS norm
+    with a weight), rotates kr and the rotated part of q (PairwiseRotary).
+    A layer built with writes_cache=False only reads: it attends over
+    the rows another layer wrote into the cache it is pointed at.
+
+    Cache per owning layer (allocated by the runner, paged by the
+    ordinary block table): [blocks, block_size, kv_rank + rot_dim]."""
+
+    def __init__(self, num_heads: int, nope_dim: int, rot_dim: int,
+                 kv_rank: int, scale: float, rotary, eps: float,
+                 cache_idx: int, writes_cache: bool = True,
+                 has_sink: bool = False):
+        super().__init__()
+        self.num_heads = num_heads
+        self.nope_dim = nope_dim
+        self.rot_dim = rot_dim
+        self.kv_rank = kv_rank
+        self.scale = scale
+        self.rotary = rotary
+        self.eps = eps
+        self.cache_idx = cache_idx
+        self.writes_cache = writes_cache
+        self.sink = (nn.Parameter(torch.zeros(num_heads,
+                                              dtype=torch.float32),
+                                  requires_grad=False)
+                     if has_sink else None)
+
+    def prepare(self, q, dkv, norm_w, positions):
+        """Rotate q's rotated part in place; norm/rotate dkv and write
+        it to the cache (when this layer owns one)."""
+        ctx = get_forward_context()
+        meta = ctx.attn_metadata
+        cache = slots = None
+        if ctx.kv_caches and self.writes_cache:
+            cache = ctx.kv_caches[self.cache_idx]
+            slots = meta.slot_mapping
+        else:
+            dkv = None
+        ops.latent_rope_cache_write(
+            q, dkv, norm_w, self.eps, positions, self.rotary.inv_freq,
+            self.nope_dim, self.kv_rank, cache, slots)
+
+    def forward(self, q_abs, q_rot) -> torch.Tensor:
+        """q_abs [T, H, kv_rank], q_rot [T, H, rot_dim] (may be a strided
+        view) -> [T, H, kv_rank]."""
+        ctx = get_forward_context()
+        meta = ctx.attn_metadata
+        if not ctx.kv_caches:
+            # Memory-profiling run: only the activation footprint counts.
+            return torch.zeros_like(q_abs)
+        return ops.latent_attention(
+            q_abs, q_rot, ctx.kv_caches[self.cache_idx], meta.block_table,
+            meta.query_start_loc, meta.seq_lens, self.scale,
+            sink=self.sink, num_decodes=meta.num_decodes,
+            max_seq_len=meta.max_seq_len,
+            max_query_len=meta.max_query_len)

@@ -40,6 +40,7 @@ class FusedMoE(nn.Module):
         enable_expert_parallel: bool = False,
         eplb_window: int = 0,
         learned_router: bool = True,
+        gated: bool = True,
     ):
         super().__init__()
         from vllm_amd.parallel.state import get_ep_group
@@ -73,9 +74,16 @@ class FusedMoE(nn.Module):
         self.gate = (ReplicatedLinear(hidden_size, num_experts, bias=False,
                                       dtype=dtype)
                      if learned_router else None)
+        # gated=False: experts are down(act(up x)) with no gate half
+        # (activation "relu2"); w13 then holds the up projection alone.
+        self.gated = gated
+        if not gated and (tp > 1 or self.ep_size > 1):
+            raise NotImplementedError(
+                "ungated experts are not sharded (tp and ep must be 1)")
         # TP: [E, 2*I/tp, H]; EP: [E/ep, 2*I, H].
         self.w13 = nn.Parameter(
-            torch.empty(self.num_local_experts, 2 * self.i_shard,
+            torch.empty(self.num_local_experts,
+                        (2 if gated else 1) * self.i_shard,
                         hidden_size, dtype=dtype),
             requires_grad=False,
         )
@@ -294,6 +302,11 @@ class FusedMoE(nn.Module):
         """Shard full expert weights onto this rank: w1/w3 [E, I, H]
         (gate / up), w2 [E, H, I]."""
         i = self.i_shard
+        if not self.gated:
+            # w1_full is unused: the up projection is the whole w13.
+            self.w13.data.copy_(w3_full)
+            self.w2.data.copy_(w2_full)
+            return
         if self.ep_size > 1:
             lo, hi = self.expert_lo, self.expert_lo + self.num_local_experts
             self.w13.data[:, :i] = w1_full[lo:hi]
@@ -304,6 +317,26 @@ class FusedMoE(nn.Module):
         self.w13.data[:, :i] = w1_full[:, r * i:(r + 1) * i]
         self.w13.data[:, i:] = w3_full[:, r * i:(r + 1) * i]
         self.w2.data.copy_(w2_full[:, :, r * i:(r + 1) * i])
+
+
+class SoftmaxTopKRouter(nn.Module):
+    """Learned router scored in fp32: softmax over ALL experts, the
+    top_k largest scores, renormalised over the chosen ones
+    (s / (sum + 1e-20)) and multiplied by `scale`. The gate weight is
+    kept in fp32 so the logits are fp32 whatever the compute dtype."""
+
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int,
+                 scale: float = 1.0):
+        super().__init__()
+        self.top_k = top_k
+        self.scale = scale
+        self.weight = nn.Parameter(
+            torch.empty(num_experts, hidden_size, dtype=torch.float32),
+            requires_grad=False)
+
+    def forward(self, hidden: torch.Tensor):
+        logits = torch.nn.functional.linear(hidden.float(), self.weight)
+        return ops.softmax_topk_scaled(logits, self.top_k, self.scale)
 
 
 class TokenTableRouter(nn.Module):

@@ -25,6 +25,19 @@ class RMSNorm(nn.Module):
             return ops.rms_norm(x, self.weight, self.eps)
         return ops.fused_add_rms_norm(x, residual, self.weight, self.eps)
 
+    def cast(self, x: torch.Tensor, out_dtype) -> torch.Tensor:
+        """Norm computed in fp32 from x of any dtype, stored as
+        out_dtype (an fp32 residual stream feeding a 16-bit GEMM)."""
+        return ops.rms_norm_cast(x, self.weight, self.eps, out_dtype)
+
+    def add_into(self, residual: torch.Tensor, y: torch.Tensor,
+                 out_dtype=None) -> torch.Tensor:
+        """Norm on a sublayer's OUTPUT: residual (fp32, in place) +=
+        norm(y) * weight in one pass; hands back the updated residual,
+        as a copy in out_dtype when the next GEMM wants 16 bits."""
+        return ops.add_rms_norm(residual, y, self.weight, self.eps,
+                                out_dtype)
+
 
 class LayerNorm(nn.Module):
     """Plain LayerNorm (OPT family). Uses torch's — not a hot op for the

@@ -126,3 +126,21 @@ class RotaryEmbedding(nn.Module):
             positions, q, k, self.cos_sin_cache, self.rotary_dim, self.is_neox
         )
         return q, k
+
+
+class PairwiseRotary(nn.Module):
+    """Rotation of adjacent coordinate pairs (2i, 2i+1), i < dims/2, of
+    a vector by the angle position * base**(-2i/dims); coordinates from
+    `dims` on pass unchanged. Angles are formed from the position itself
+    in fp32 inside the kernels that apply the rotation (no table, so no
+    bound on the context); this module only owns the frequency row."""
+
+    def __init__(self, dims: int, base: float):
+        super().__init__()
+        assert dims % 2 == 0
+        self.dims = dims
+        self.base = float(base)
+        freq = [self.base ** (-2.0 * i / dims) for i in range(dims // 2)]
+        self.register_buffer(
+            "inv_freq", torch.tensor(freq, dtype=torch.float32),
+            persistent=False)

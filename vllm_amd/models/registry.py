@@ -53,6 +53,10 @@ def get_model_class(architecture: str):
         from vllm_amd.models.gadilix import GadilixForCausalLM
 
         return GadilixForCausalLM
+    if architecture == "papunex":
+        from vllm_amd.models.papunex import PapunexForCausalLM
+
+        return PapunexForCausalLM
     if architecture == "deepseek":
         from vllm_amd.models.deepseek import DeepseekForCausalLM
 

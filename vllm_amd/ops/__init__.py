@@ -223,3 +223,73 @@ def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
 
 
 from vllm_amd.ops._torch_ref import pool_slots_per_page  # noqa: E402,F401
+
+
+# ---------------------------------------------------------------------
+# fp32 residual stream with weighted output norms, latent attention with
+# a softmax sink, state-space-duality mixers, squared-relu experts (see
+# _torch_ref.py for semantics).
+
+def scaled_embedding(input_ids, table, scale):
+    return get_backend(table.device).scaled_embedding(input_ids, table,
+                                                      scale)
+
+
+def rms_norm_cast(x, weight, eps, out_dtype):
+    return get_backend(x.device).rms_norm_cast(x, weight, eps, out_dtype)
+
+
+def add_rms_norm(residual, y, weight, eps, out_dtype=None):
+    return get_backend(residual.device).add_rms_norm(
+        residual, y, weight, eps, out_dtype)
+
+
+def relu2(x):
+    return get_backend(x.device).relu2(x)
+
+
+def logit_softcap(logits, cap):
+    return get_backend(logits.device).logit_softcap(logits, cap)
+
+
+def softmax_topk_scaled(logits, topk, scale):
+    return get_backend(logits.device).softmax_topk_scaled(logits, topk,
+                                                          scale)
+
+
+def latent_rope_cache_write(q, dkv, norm_w, eps, positions, inv_freq,
+                            nope_dim, kv_rank, cache, slot_mapping):
+    return get_backend(q.device).latent_rope_cache_write(
+        q, dkv, norm_w, eps, positions, inv_freq, nope_dim, kv_rank,
+        cache, slot_mapping)
+
+
+def latent_attention(q_abs, q_rot, cache, block_table, query_start_loc,
+                     seq_lens, scale, sink=None, num_decodes=0,
+                     max_seq_len=0, max_query_len=0):
+    return get_backend(q_abs.device).latent_attention(
+        q_abs, q_rot, cache, block_table, query_start_loc, seq_lens, scale,
+        sink, num_decodes, max_seq_len, max_query_len)
+
+
+def sigmoid_gate_mul(x, gate):
+    return get_backend(x.device).sigmoid_gate_mul(x, gate)
+
+
+def causal_conv_silu(x, weight, bias, conv_state, state_rows,
+                     query_start_loc, out_dtype=None):
+    return get_backend(x.device).causal_conv_silu(
+        x, weight, bias, conv_state, state_rows, query_start_loc,
+        out_dtype)
+
+
+def ssd_scan(xbc, heads, head_dim, groups, state, dt, dt_bias, a_log,
+             d_skip, ssm_state, state_rows, query_start_loc):
+    return get_backend(xbc.device).ssd_scan(
+        xbc, heads, head_dim, groups, state, dt, dt_bias, a_log, d_skip,
+        ssm_state, state_rows, query_start_loc)
+
+
+def gated_group_rms_norm(y, z, weight, eps, groups, out_dtype):
+    return get_backend(y.device).gated_group_rms_norm(
+        y, z, weight, eps, groups, out_dtype)

@@ -196,12 +196,14 @@ def fused_moe(hidden, w13, w2, topk_weights, topk_ids, activation="silu"):
     """Reference MoE: loop over experts.
 
     hidden: [T, H]; w13: [E, 2I, H]; w2: [E, H, I];
-    topk_weights/topk_ids: [T, k]. Returns [T, H].
+    topk_weights/topk_ids: [T, k]. Returns [T, H]. activation "relu2"
+    is not gated: w13 is the up projection alone, [E, I, H].
     """
     T, H = hidden.shape
     E = w13.shape[0]
     out = torch.zeros(T, H, dtype=torch.float32, device=hidden.device)
-    act = silu_and_mul if activation == "silu" else gelu_and_mul
+    act = {"silu": silu_and_mul, "gelu": gelu_and_mul,
+           "relu2": relu2}[activation]
     flat_ids = topk_ids.long()
     for e in range(E):
         mask = flat_ids == e  # [T, k]
@@ -467,3 +469,211 @@ def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
                 o = o * torch.sigmoid(gate[s + t].float()).unsqueeze(-1)
             out[s + t] = o.to(out.dtype)
     return out
+
+
+# ---------------------------------------------------------------------
+# fp32 residual stream with weighted output norms, latent attention
+# with a softmax sink over a shared latent cache, state-space-duality
+# (Mamba-2) mixers, squared-relu experts.
+
+def scaled_embedding(input_ids, table, scale):
+    """fp32 rows table[id] * scale."""
+    return table[input_ids].float() * scale
+
+
+def rms_norm_cast(x, weight, eps, out_dtype):
+    """x / sqrt(mean(x^2) + eps) * w in fp32, stored as out_dtype."""
+    xf = x.float()
+    inv = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * inv * weight.float()).to(out_dtype)
+
+
+def add_rms_norm(residual, y, weight, eps, out_dtype=None):
+    """residual (fp32, in place) += norm(y) * w. Returns the updated
+    residual, as a copy in out_dtype when that is a 16-bit type."""
+    yf = y.float()
+    inv = torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
+    residual.add_(yf * inv * weight.float())
+    if out_dtype is None or out_dtype == torch.float32:
+        return residual
+    return residual.to(out_dtype)
+
+
+def relu2(x):
+    r = torch.relu(x)
+    return r * r
+
+
+def logit_softcap(logits, cap):
+    return cap * torch.tanh(logits.float() / cap)
+
+
+def softmax_topk_scaled(logits, topk, scale):
+    """Softmax over all experts (fp32), the topk largest, each divided
+    by their sum (+1e-20) and multiplied by scale."""
+    probs = logits.float().softmax(dim=-1)
+    w, ids = probs.topk(topk, dim=-1)
+    w = w / (w.sum(dim=-1, keepdim=True) + 1e-20) * scale
+    return w, ids.to(torch.int32)
+
+
+def _rotate_pairs(v, positions, inv_freq):
+    """v [T, ..., n] float; pairs (2i, 2i+1) for i < len(inv_freq) turn
+    by positions * inv_freq[i]; the remaining coordinates pass."""
+    n2 = inv_freq.shape[0] * 2
+    if n2 == 0:
+        return v
+    ang = positions.float().unsqueeze(-1) * inv_freq.float()
+    shape = [v.shape[0]] + [1] * (v.dim() - 2) + [n2 // 2]
+    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    u, w = v[..., 0:n2:2], v[..., 1:n2:2]
+    out = v.clone()
+    out[..., 0:n2:2] = u * c - w * s
+    out[..., 1:n2:2] = w * c + u * s
+    return out
+
+
+def latent_rope_cache_write(q, dkv, norm_w, eps, positions, inv_freq,
+                            nope_dim, kv_rank, cache, slot_mapping):
+    """q [T, H, nope+rot] (modified in place): the last rot coordinates
+    of every head are rotated. dkv [T, kv_rank+rot] or None: the first
+    kv_rank coordinates are RMS-normed (weight norm_w), the rest
+    rotated, and the row is written to cache [blocks, page, kv_rank+rot]
+    at slot_mapping (negative slots are skipped)."""
+    qr = q[..., nope_dim:]
+    qr.copy_(_rotate_pairs(qr.float(), positions, inv_freq).to(q.dtype))
+    if dkv is None:
+        return
+    d = dkv.float()
+    c = d[:, :kv_rank]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) \
+        * norm_w.float()
+    kr = _rotate_pairs(d[:, kv_rank:], positions, inv_freq)
+    row = torch.cat([c, kr], dim=-1).to(cache.dtype)
+    ok = slot_mapping >= 0
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping[ok]] = row[ok]
+
+
+def latent_attention(q_abs, q_rot, cache, block_table, query_start_loc,
+                     seq_lens, scale, sink=None, num_decodes=0,
+                     max_seq_len=0, max_query_len=0):
+    """Causal attention of every head over ONE shared latent stream.
+    q_abs [T, H, L] (queries already carried into the latent space),
+    q_rot [T, H, R], cache [blocks, page, L+R]; score = (q_abs . c +
+    q_rot . kr) * scale; value = c. sink [H] adds exp(sink_h) to the
+    softmax denominator (no key, no value, not scaled). -> [T, H, L]."""
+    T, H, L = q_abs.shape
+    page = cache.shape[1]
+    out = torch.zeros(T, H, L, dtype=q_abs.dtype, device=q_abs.device)
+    qsl = query_start_loc.tolist()
+    lens = seq_lens.tolist()
+    for r in range(len(lens)):
+        s, e = qsl[r], qsl[r + 1]
+        n, ctx = e - s, lens[r]
+        if n == 0 or ctx == 0:
+            continue
+        nb = -(-ctx // page)
+        rows = cache[block_table[r, :nb].long()].reshape(
+            nb * page, -1)[:ctx].float()
+        c, kr = rows[:, :L], rows[:, L:]
+        sc = (torch.einsum("nhl,kl->hnk", q_abs[s:e].float(), c)
+              + torch.einsum("nhr,kr->hnk", q_rot[s:e].float(), kr)) * scale
+        pos = torch.arange(ctx - n, ctx, device=sc.device)
+        hide = torch.arange(ctx, device=sc.device)[None, :] > pos[:, None]
+        sc = sc.masked_fill(hide[None], float("-inf"))
+        if sink is not None:
+            extra = sink.float().view(H, 1, 1).expand(H, n, 1)
+            p = torch.cat([sc, extra], dim=-1).softmax(dim=-1)[..., :ctx]
+        else:
+            p = sc.softmax(dim=-1)
+        out[s:e] = torch.einsum("hnk,kl->nhl", p, c).to(out.dtype)
+    return out
+
+
+def sigmoid_gate_mul(x, gate):
+    """x [T, H, D] (any strides) * sigmoid(gate [T, H*D]) ->
+    contiguous [T, H*D]."""
+    xf = x.reshape(x.shape[0], -1).float()
+    return (xf * torch.sigmoid(gate.float())).to(x.dtype).contiguous()
+
+
+def causal_conv_silu(x, weight, bias, conv_state, state_rows,
+                     query_start_loc, out_dtype=None):
+    """Per-channel causal convolution + silu over a varlen batch.
+    x [T, C]; weight [C, K] (last tap = current token); conv_state
+    [rows, C, K-1] holds each request's last K-1 inputs (oldest first)
+    and is advanced in place; None = zero history, nothing kept.
+    Returns a contiguous [T, C] in out_dtype (default: x's)."""
+    T, C = x.shape
+    K = weight.shape[1]
+    out = torch.empty(T, C, dtype=out_dtype or x.dtype, device=x.device)
+    qsl = query_start_loc.tolist()
+    wf, bf = weight.float(), bias.float()
+    for r in range(len(qsl) - 1):
+        s, e = qsl[r], qsl[r + 1]
+        if s == e:
+            continue
+        if conv_state is not None:
+            row = int(state_rows[r])
+            hist = conv_state[row].float()
+        else:
+            hist = torch.zeros(C, K - 1, device=x.device)
+        ext = torch.cat([hist, x[s:e].float().t()], dim=1)  # [C, K-1+n]
+        if conv_state is not None and K > 1:
+            conv_state[row] = ext[:, ext.shape[1] - (K - 1):].to(
+                conv_state.dtype)
+        win = ext.unfold(1, K, 1)                           # [C, n, K]
+        y = (win * wf[:, None, :]).sum(-1) + bf[:, None]
+        out[s:e] = (y * torch.sigmoid(y)).t().to(out.dtype)
+    return out
+
+
+def ssd_scan(xbc, heads, head_dim, groups, state, dt, dt_bias, a_log,
+             d_skip, ssm_state, state_rows, query_start_loc):
+    """State-space-duality recurrence per head over a varlen batch.
+    xbc [T, heads*head_dim + 2*groups*state] = x | B | C; dt [T, heads]
+    (raw); ssm_state [rows, heads, head_dim, state] fp32 advanced in
+    place (None = zero start). Head h uses B/C group h // (heads/groups).
+      dt' = softplus(dt + dt_bias);  S <- exp(-exp(a_log) dt') S
+      + dt' x B^T;  y = S C + d_skip x.     -> y fp32 [T, heads, head_dim]"""
+    T = xbc.shape[0]
+    Hm, P, G, N = heads, head_dim, groups, state
+    inner = Hm * P
+    per = Hm // G
+    xf = xbc[:, :inner].float().view(T, Hm, P)
+    Bh = xbc[:, inner:inner + G * N].float().view(
+        T, G, N).repeat_interleave(per, dim=1)                 # [T, Hm, N]
+    Ch = xbc[:, inner + G * N:].float().view(
+        T, G, N).repeat_interleave(per, dim=1)
+    y = torch.empty(T, Hm, P, dtype=torch.float32, device=xbc.device)
+    dtp = torch.nn.functional.softplus(dt.float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * dtp)        # [T, Hm]
+    qsl = query_start_loc.tolist()
+    for r in range(len(qsl) - 1):
+        s, e = qsl[r], qsl[r + 1]
+        if s == e:
+            continue
+        if ssm_state is not None:
+            row = int(state_rows[r])
+            S = ssm_state[row].clone()
+        else:
+            S = torch.zeros(Hm, P, N, device=xbc.device)
+        for t in range(s, e):
+            S = decay[t, :, None, None] * S + dtp[t, :, None, None] * (
+                xf[t, :, :, None] * Bh[t, :, None, :])
+            y[t] = (S * Ch[t, :, None, :]).sum(-1)
+        if ssm_state is not None:
+            ssm_state[row] = S
+    return y + d_skip.float()[None, :, None] * xf
+
+
+def gated_group_rms_norm(y, z, weight, eps, groups, out_dtype):
+    """(y * silu(z)) normed in `groups` equal parts, each by its own
+    root mean square, times weight. y fp32 [T, W], z [T, W]."""
+    T, W = y.shape
+    zf = z.float()
+    g = y.float() * (zf * torch.sigmoid(zf))
+    g = g.view(T, groups, W // groups)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+    return (g.reshape(T, W) * weight.float()).to(out_dtype)

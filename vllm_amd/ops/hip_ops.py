@@ -330,7 +330,8 @@ def fused_moe(hidden, w13, w2, topk_weights, topk_ids, activation="silu",
     x = hidden[token_of].contiguous()
     out_sorted = torch.empty(T * k, H, dtype=hidden.dtype,
                              device=hidden.device)
-    act = silu_and_mul if activation == "silu" else gelu_and_mul
+    act = {"silu": silu_and_mul, "gelu": gelu_and_mul,
+           "relu2": lambda v: _C.relu2(v.contiguous())}[activation]
     offset = 0
     for e in range(E):
         c = counts[e]
@@ -429,3 +430,71 @@ def pooled_window_attention(q, k_cache, v_cache, pool_k, pool_v,
             query_start_loc, seq_lens, gate, scale, window, pool,
             num_decodes, max_query_len)
     return out
+
+
+# ---------------------------------------------------------------------
+# fp32 residual stream with weighted output norms (csrc/residual_ops.hip),
+# latent attention with a softmax sink (csrc/latent_attention*.hip),
+# state-space-duality mixers (csrc/ssd.hip).
+
+from vllm_amd.ops._torch_ref import softmax_topk_scaled  # noqa: E402,F401
+
+
+def scaled_embedding(input_ids, table, scale):
+    return _C.scaled_embedding(input_ids.contiguous(), table, float(scale))
+
+
+def rms_norm_cast(x, weight, eps, out_dtype):
+    return _C.rms_norm_cast(x.contiguous(), weight, eps, out_dtype)
+
+
+def add_rms_norm(residual, y, weight, eps, out_dtype=None):
+    return _C.add_rms_norm(residual, y.contiguous(), weight, eps, out_dtype)
+
+
+def relu2(x):
+    return _C.relu2(x.contiguous())
+
+
+def logit_softcap(logits, cap):
+    return _C.logit_softcap(logits.contiguous(), float(cap))
+
+
+def sigmoid_gate_mul(x, gate):
+    return _C.sigmoid_gate_mul(x, gate)
+
+
+def latent_rope_cache_write(q, dkv, norm_w, eps, positions, inv_freq,
+                            nope_dim, kv_rank, cache, slot_mapping):
+    _C.latent_rope_cache_write(q, dkv, norm_w, eps, positions, inv_freq,
+                               nope_dim, kv_rank, cache, slot_mapping)
+
+
+def latent_attention(q_abs, q_rot, cache, block_table, query_start_loc,
+                     seq_lens, scale, sink=None, num_decodes=0,
+                     max_seq_len=0, max_query_len=0):
+    T, H, L = q_abs.shape
+    out = torch.empty(T, H, L, dtype=q_abs.dtype, device=q_abs.device)
+    _C.latent_attention_rows(out, q_abs, q_rot, cache, block_table,
+                             query_start_loc, seq_lens, sink, scale)
+    return out
+
+
+def causal_conv_silu(x, weight, bias, conv_state, state_rows,
+                     query_start_loc, out_dtype=None):
+    return _C.causal_conv_silu(
+        x, weight, bias, conv_state,
+        state_rows if conv_state is not None else None, query_start_loc,
+        out_dtype or x.dtype)
+
+
+def ssd_scan(xbc, heads, head_dim, groups, state, dt, dt_bias, a_log,
+             d_skip, ssm_state, state_rows, query_start_loc):
+    return _C.ssd_scan(
+        xbc, heads, head_dim, groups, state, dt.float(), dt_bias, a_log,
+        d_skip, ssm_state,
+        state_rows if ssm_state is not None else None, query_start_loc)
+
+
+def gated_group_rms_norm(y, z, weight, eps, groups, out_dtype):
+    return _C.gated_group_rms_norm(y, z, weight, eps, groups, out_dtype)

@@ -66,6 +66,11 @@ class ForwardContext:
     # token's mixer input per running request and layer, indexed by
     # attn_metadata.state_rows; None during memory profiling.
     shift_states: Optional[torch.Tensor] = None
+    # Layer-listed stacks with recurrent layers: one entry per such
+    # layer, (conv tail [rows, channels, taps-1], recurrent state
+    # [rows, heads, N, head_dim] fp32), indexed by
+    # attn_metadata.state_rows; None during memory profiling.
+    layer_states: Optional[list] = None
     # Encoder-decoder (whisper): per-request cached audio-encoder
     # states, in this batch's request order ([T_audio, H] tensors or
     # None for requests without audio / padded rows).

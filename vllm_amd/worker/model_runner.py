@@ -129,7 +129,8 @@ class DecodeGraphRunner:
                                         dtype=torch.int32, pin_memory=True)
         # Row-state models (token-shift carry): the state row of each
         # batch entry; padded entries point at the scratch row.
-        self.row_state = runner.spec.has_token_shift
+        self.row_state = (runner.spec.has_token_shift
+                          or runner.spec.has_layer_state)
         self.scratch_row = cfg.scheduler_config.max_num_seqs
         if self.row_state:
             self.state_rows = torch.full((n,), self.scratch_row,
@@ -178,7 +179,8 @@ class DecodeGraphRunner:
         ctx = ForwardContext(attn_metadata=self._meta(nb, parts),
                              kv_caches=runner.kv_caches,
                              sp_size=self.sp_size,
-                             shift_states=runner.shift_states)
+                             shift_states=runner.shift_states,
+                             layer_states=runner.layer_states)
         if self.row_state:
             # The warmup pass below must not touch a live request's row.
             self.state_rows[:nb].fill_(self.scratch_row)
@@ -299,6 +301,9 @@ class ModelRunner:
         # scratch row last, cleared on (re)admission).
         self.has_row_state = self.spec.has_row_state
         self.shift_states: Optional[torch.Tensor] = None
+        # Layer-listed stacks: (conv tail, recurrent state) per
+        # recurrent layer, rows as above.
+        self.layer_states: Optional[list] = None
         self.np_block_table_w = (np.zeros((n, mb), dtype=np.int32)
                                  if self.mixed_attn else None)
         self.np_nblocks = np.zeros(n, dtype=np.int32)
@@ -454,6 +459,19 @@ class ModelRunner:
             # the profiled pool lands at a sane size (state tensors are
             # tiny and allocated separately in allocate_kv_cache).
             return self.block_size * 2 * spec.hidden_size * elt
+        if spec.architecture == "papunex":
+            # One latent row per token and key-owning layer; layers
+            # that read another layer's keys and recurrent layers add
+            # nothing. A stack without attention prices a block like
+            # the pure-SSM case above.
+            per_tok = sum(
+                int(e["mixer"]["kv_rank"]) + int(e["mixer"]["rot_dim"])
+                for e in spec.layer_specs
+                if e["type"] == "latent_attention"
+                and e["mixer"].get("kv_from") is None)
+            if per_tok == 0:
+                return self.block_size * 2 * spec.hidden_size * elt
+            return self.block_size * per_tok * elt
         if spec.layer_specs is not None:
             # Per-layer geometry: K and V widths differ, and windowed
             # layers with pooled far blocks add an fp32 pooled area.
@@ -498,6 +516,39 @@ class ModelRunner:
             self.shift_states = torch.zeros(
                 spec.num_layers, rows, spec.hidden_size,
                 dtype=torch.float32, device=self.device)
+        if spec.architecture == "papunex":
+            # Indexed by layer: a key-owning latent layer gets a paged
+            # [blocks, page, kv_rank + rot_dim] cache, a layer that
+            # reads another's keys shares that tensor, a recurrent
+            # layer has none and keeps (conv tail, fp32 state) rows
+            # instead, one scratch row last for padded entries.
+            from vllm_amd.layers.mamba2 import Mamba2Mixer
+            rows = self.config.scheduler_config.max_num_seqs + 1
+            self.kv_caches = []
+            self.layer_states = []
+            for entry in spec.layer_specs:
+                mx = entry["mixer"]
+                if entry["type"] == "mamba2":
+                    conv_shape, ssm_shape = Mamba2Mixer.state_shapes(mx)
+                    self.layer_states.append((
+                        torch.zeros((rows,) + conv_shape, dtype=self.dtype,
+                                    device=self.device),
+                        torch.zeros((rows,) + ssm_shape,
+                                    dtype=torch.float32,
+                                    device=self.device)))
+                    self.kv_caches.append(None)
+                elif mx.get("kv_from") is not None:
+                    self.kv_caches.append(
+                        self.kv_caches[int(mx["kv_from"])])
+                else:
+                    self.kv_caches.append(torch.zeros(
+                        num_blocks, self.block_size,
+                        int(mx["kv_rank"]) + int(mx["rot_dim"]),
+                        dtype=self.dtype, device=self.device))
+            if not self.layer_states:
+                self.layer_states = None
+            self.graph_runner = None
+            return
         if spec.layer_specs is not None:
             # One (k, v, pooled k, pooled v) tuple per layer RUN — layers
             # that borrow another layer's weights still cache their own
@@ -752,6 +803,13 @@ class ModelRunner:
         if self.num_host_blocks:
             self.allocate_host_kv_pool(self.num_host_blocks)
 
+    def _clear_layer_states(self, row: int) -> None:
+        """A row handed to a (re)admitted request starts from zero."""
+        if self.layer_states is not None:
+            for conv, ssm in self.layer_states:
+                conv[row] = 0
+                ssm[row] = 0
+
     # ------------------------------------------------------------------
     def _update_states(self, so: SchedulerOutput) -> None:
         if (self._eplb_every and so.total_num_scheduled_tokens > 0
@@ -798,6 +856,7 @@ class ModelRunner:
                 self.mamba_ssm[:, row] = 0
             if self.shift_states is not None:
                 self.shift_states[:, row] = 0
+            self._clear_layer_states(row)
             nb = len(nr.block_ids)
             self.np_block_table[row, :nb] = nr.block_ids
             if self.mixed_attn and nr.block_ids_w:
@@ -834,6 +893,7 @@ class ModelRunner:
                     self.mamba_ssm[:, row] = 0
                 if self.shift_states is not None:
                     self.shift_states[:, row] = 0
+                self._clear_layer_states(row)
                 state.block_ids = list(cr.new_block_ids[i])
                 state.token_ids = list(cr.new_token_ids[i])
                 if state.prompt_open:
@@ -1041,6 +1101,7 @@ class ModelRunner:
                 mamba_states=((self.mamba_conv, self.mamba_ssm)
                               if self.is_mamba else None),
                 shift_states=self.shift_states,
+                layer_states=self.layer_states,
                 cross_feats=cross,
             )
             with set_forward_context(ctx):
@@ -1399,6 +1460,7 @@ class ModelRunner:
             mamba_states=((self.mamba_conv, self.mamba_ssm)
                           if self.is_mamba else None),
             shift_states=self.shift_states,
+                layer_states=self.layer_states,
             cross_feats=cross_feats,
         )
         if self.pp_size > 1:
