@@ -63,9 +63,7 @@ def latent_attention(h, mx, W, pre, eps, shared=None):
             qn = q[t, hh, :D]
             qr = rotate_pairs(q[t, hh, D:], t, mx["rot"]["base"],
                               mx["rot"]["dims"])
-            s = torch.stack([
-                (qn @ k_nope[j, hh] + qr @ kr[j]) * mx["scale"]
-                for j in range(t + 1)])
+            s = (k_nope[:t + 1, hh] @ qn + kr[:t + 1] @ qr) * mx["scale"]
             m = max(float(s.max()), float(sink[hh]))
             e = torch.exp(s - m)
             den = e.sum() + math.exp(float(sink[hh]) - m)
@@ -185,3 +183,131 @@ def forward(cfg, W, tokens, return_layers=False):
     if cap:
         logits = cap * torch.tanh(logits / cap)
     return (logits, torch.stack(per_layer)) if return_layers else logits
+
+
+# ---------------------------------------------------------------------
+# Test models: configurations, random weights, files on disk.
+
+def latent_entry(heads=2, dim=8, rot_dim=4, vdim=8, kv_rank=8,
+                 rot_dims=None, base=100.0, scale=None, kv_from=None,
+                 mlp="dense", ff=16, experts=4, top=2, router_scale=1.0,
+                 shared_ff=8):
+    mx = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim,
+          "kv_rank": kv_rank,
+          "rot": {"base": base,
+                  "dims": rot_dim if rot_dims is None else rot_dims},
+          "scale": scale if scale is not None
+          else 1.0 / math.sqrt(dim + rot_dim)}
+    if kv_from is not None:
+        mx["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": mx,
+            "mlp": mlp_entry(mlp, ff, experts, top, router_scale,
+                             shared_ff)}
+
+
+def mamba_entry(heads=4, vdim=8, state=8, groups=2, conv=4, norm_groups=2,
+                mlp="dense", ff=16, experts=4, top=2, router_scale=1.0,
+                shared_ff=8):
+    mx = {"heads": heads, "vdim": vdim, "state": state, "groups": groups,
+          "conv": conv, "norm_groups": norm_groups}
+    return {"type": "mamba2", "mixer": mx,
+            "mlp": mlp_entry(mlp, ff, experts, top, router_scale,
+                             shared_ff)}
+
+
+def mlp_entry(kind, ff, experts, top, router_scale, shared_ff):
+    if kind is None:
+        return None
+    if kind == "dense":
+        return {"kind": "dense", "ff": ff}
+    out = {"kind": "moe", "expert": {"ff": ff},
+           "router": {"experts": experts, "top": top,
+                      "scale": router_scale}}
+    if shared_ff:
+        out["shared"] = {"ff": shared_ff}
+    return out
+
+
+def make_config(layers, vocab=48, width=24, eps=1e-5, embed_scale=2.0,
+                softcap=20.0):
+    return {"architecture": "Papunex", "vocab": vocab, "width": width,
+            "embedding": {"scale": embed_scale}, "norm": {"eps": eps},
+            "logit_softcap": softcap, "layers": layers}
+
+
+def random_weights(cfg, seed=0):
+    """fp32 tensors whose values are exactly representable in bf16."""
+    gen = torch.Generator().manual_seed(seed)
+    Wd = cfg["width"]
+
+    def mat(o, i, gain=1.0):
+        w = torch.randn(o, i, generator=gen) * gain / math.sqrt(i)
+        return w.bfloat16().float()
+
+    def vec(n, lo, hi):
+        return (torch.rand(n, generator=gen) * (hi - lo) + lo) \
+            .bfloat16().float()
+
+    W = {"embed": (torch.randn(cfg["vocab"], Wd, generator=gen) * 0.5)
+         .bfloat16().float(),
+         "final.norm": vec(Wd, 0.5, 1.5),
+         "head": mat(cfg["vocab"], Wd, 2.0)}
+    for i, lay in enumerate(cfg["layers"]):
+        mx, pre = lay["mixer"], f"l{i}.mix."
+        W[f"l{i}.norm1"] = vec(Wd, 0.5, 1.5)
+        if lay["type"] == "latent_attention":
+            H, D, R = mx["heads"], mx["dim"], mx["rot_dim"]
+            Dv, L = mx["vdim"], mx["kv_rank"]
+            W[pre + "q"] = mat(H * (D + R), Wd, 2.0)
+            if mx.get("kv_from") is None:
+                W[pre + "dkv"] = mat(L + R, Wd, 2.0)
+                W[pre + "dkv.norm"] = vec(L, 0.5, 1.5)
+            W[pre + "uk"] = mat(H * D, L, 2.0)
+            W[pre + "uv"] = mat(H * Dv, L)
+            W[pre + "sink"] = vec(H, -1.0, 2.0)
+            W[pre + "g"] = mat(H * Dv, Wd)
+            W[pre + "o"] = mat(Wd, H * Dv)
+        else:
+            Hm, P, N, G = (mx["heads"], mx["vdim"], mx["state"],
+                           mx["groups"])
+            inner, ch = Hm * P, Hm * P + 2 * G * N
+            W[pre + "in"] = mat(2 * inner + 2 * G * N + Hm, Wd)
+            W[pre + "conv"] = mat(ch, mx["conv"], 1.5)
+            W[pre + "conv.b"] = vec(ch, -0.2, 0.2)
+            W[pre + "dt_bias"] = vec(Hm, -2.0, 0.5)
+            W[pre + "A_log"] = vec(Hm, -1.5, 0.5)
+            W[pre + "D"] = vec(Hm, 0.5, 1.5)
+            W[pre + "norm"] = vec(inner, 0.5, 1.5)
+            W[pre + "o"] = mat(Wd, inner)
+        ml = lay.get("mlp")
+        if ml is None:
+            continue
+        W[f"l{i}.norm2"] = vec(Wd, 0.5, 1.5)
+        pre = f"l{i}.mlp."
+        if ml["kind"] == "dense":
+            W[pre + "up"] = mat(ml["ff"], Wd, 1.5)
+            W[pre + "down"] = mat(Wd, ml["ff"], 1.5)
+            continue
+        W[pre + "router"] = mat(ml["router"]["experts"], Wd, 3.0)
+        for e in range(ml["router"]["experts"]):
+            W[f"{pre}e{e}.up"] = mat(ml["expert"]["ff"], Wd, 1.5)
+            W[f"{pre}e{e}.down"] = mat(Wd, ml["expert"]["ff"], 1.5)
+        if ml.get("shared"):
+            W[pre + "shared.up"] = mat(ml["shared"]["ff"], Wd, 1.5)
+            W[pre + "shared.down"] = mat(Wd, ml["shared"]["ff"], 1.5)
+            W[pre + "shared.sg"] = mat(1, Wd, 2.0)
+    return W
+
+
+def save_model(path, cfg, W):
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.bfloat16().contiguous() for k, v in W.items()},
+              os.path.join(path, "model.safetensors"))
+    return path
