@@ -33,6 +33,7 @@ SOURCES = [
     CSRC / "pooled_attention_decode.hip",
     CSRC / "residual_ops.hip",
     CSRC / "latent_attention.hip",
+    CSRC / "latent_attention_tiles.hip",
     CSRC / "ssd.hip",
     CSRC / "gemm_hipblaslt.cpp",
     CSRC / "bindings.cpp",

@@ -118,6 +118,14 @@ void latent_attention_rows(torch::Tensor out, torch::Tensor q_abs,
                            torch::Tensor query_start_loc,
                            torch::Tensor seq_lens,
                            c10::optional<torch::Tensor> sink, double scale);
+bool latent_attention_tiles_supported(int64_t kv_rank, int64_t rot_dim);
+void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
+                            torch::Tensor q_rot, torch::Tensor cache,
+                            torch::Tensor block_table,
+                            torch::Tensor query_start_loc,
+                            torch::Tensor seq_lens,
+                            c10::optional<torch::Tensor> sink, double scale,
+                            int64_t num_decodes, int64_t max_seq_len);
 torch::Tensor causal_conv_silu(torch::Tensor x, torch::Tensor weight,
                                torch::Tensor bias,
                                c10::optional<torch::Tensor> conv_state,
@@ -227,6 +235,13 @@ TORCH_LIBRARY(vllm_amd, m) {
   m.def("latent_attention_rows(Tensor(a!) out, Tensor q_abs, Tensor q_rot, "
         "Tensor cache, Tensor block_table, Tensor query_start_loc, "
         "Tensor seq_lens, Tensor? sink, float scale) -> ()");
+  m.def("latent_attention_tiles_supported(int kv_rank, int rot_dim) -> bool");
+  m.impl("latent_attention_tiles_supported",
+         &vllm_amd::latent_attention_tiles_supported);
+  m.def("latent_attention_tiles(Tensor(a!) out, Tensor q_abs, Tensor q_rot, "
+        "Tensor cache, Tensor block_table, Tensor query_start_loc, "
+        "Tensor seq_lens, Tensor? sink, float scale, int num_decodes, "
+        "int max_seq_len) -> ()");
   m.def("causal_conv_silu(Tensor x, Tensor weight, Tensor bias, "
         "Tensor(a!)? conv_state, Tensor? state_rows, "
         "Tensor query_start_loc, ScalarType out_dtype) -> Tensor");
@@ -296,6 +311,7 @@ TORCH_LIBRARY_IMPL(vllm_amd, CUDA, m) {
   m.impl("sigmoid_gate_mul", &vllm_amd::sigmoid_gate_mul);
   m.impl("latent_rope_cache_write", &vllm_amd::latent_rope_cache_write);
   m.impl("latent_attention_rows", &vllm_amd::latent_attention_rows);
+  m.impl("latent_attention_tiles", &vllm_amd::latent_attention_tiles);
   m.impl("causal_conv_silu", &vllm_amd::causal_conv_silu);
   m.impl("ssd_scan", &vllm_amd::ssd_scan);
   m.impl("gated_group_rms_norm", &vllm_amd::gated_group_rms_norm);

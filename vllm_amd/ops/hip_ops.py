@@ -473,8 +473,31 @@ def latent_rope_cache_write(q, dkv, norm_w, eps, positions, inv_freq,
 def latent_attention(q_abs, q_rot, cache, block_table, query_start_loc,
                      seq_lens, scale, sink=None, num_decodes=0,
                      max_seq_len=0, max_query_len=0):
+    """bf16 batches whose (kv_rank, rot_dim) the MFMA tile kernel is
+    built for run there (prefill chunks and decode rows alike); every
+    other dtype and shape runs on the row-wise kernel, which
+    VLLM_AMD_LATENT_ROWWISE=1 forces for all."""
+    import os
+
     T, H, L = q_abs.shape
+    R = q_rot.shape[2]
     out = torch.empty(T, H, L, dtype=q_abs.dtype, device=q_abs.device)
+    if (q_abs.dtype == torch.bfloat16
+            and _C.latent_attention_tiles_supported(L, R)
+            and os.environ.get("VLLM_AMD_LATENT_ROWWISE", "0") != "1"):
+        def aligned(t):
+            return (t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0
+                    and t.storage_offset() % 8 == 0 and t.stride(2) == 1)
+        if not aligned(q_abs):
+            q_abs = q_abs.contiguous()
+        if not aligned(q_rot):
+            q_rot = q_rot.contiguous()
+        if max_seq_len <= 0:
+            max_seq_len = int(seq_lens.max().item())
+        _C.latent_attention_tiles(out, q_abs, q_rot, cache, block_table,
+                                  query_start_loc, seq_lens, sink, scale,
+                                  num_decodes, max_seq_len)
+        return out
     _C.latent_attention_rows(out, q_abs, q_rot, cache, block_table,
                              query_start_loc, seq_lens, sink, scale)
     return out
