@@ -59,7 +59,7 @@ def parse_args():
                         "scaling, xGMI-free — the throughput-optimal "
                         "serving layout for an 8B model)")
     p.add_argument("--compare-family", type=str, default=None,
-                   choices=["gadilix"],
+                   choices=["gadilix", "papunex"],
                    help="instead of the flagship workload: prefill and "
                         "decode throughput of this family beside the "
                         "closest existing one at equal active size "

@@ -2,8 +2,16 @@
 existing family at equal active size (random weights, one GPU).
 
     python bench.py --compare-family gadilix [--compare-sizes small,medium]
+    python bench.py --compare-family papunex [--compare-sizes small,medium]
 
-For every size it builds two engines in turn — the Gadilix stack
+"papunex" builds three engines per size: an all-latent-attention
+Papunex stack, a hybrid one (latent attention and Mamba-2 layers
+alternating) and a DeepSeek-structured stack (latent attention of the
+same kv_rank / rotated width / head sizes, routed SwiGLU experts plus a
+shared one) whose expert width is 2/3 of the squared-relu experts', so
+both move the same number of expert parameters per token.
+
+For every "gadilix" size it builds two engines in turn — the Gadilix stack
 (sliding window + pooled far blocks, token-table MoE + shared expert)
 and a Mixtral-structured stack (GQA attention with the same sliding
 window, learned-router MoE) whose per-token active expert width matches
@@ -38,6 +46,66 @@ SIZES = {
                    experts=8, top=2, ff=2048, window=2048, pool=64,
                    vocab=32000),
 }
+
+
+PAPUNEX_SIZES = {
+    # Latent attention with the usual 512 + 64 cache row; Mamba-2 layers
+    # of inner width 2 * width, 64-wide heads, state 128.
+    "small": dict(width=2048, layers=4, heads=16, dim=128, rot_dim=64,
+                  vdim=128, kv_rank=512, experts=8, top=2, ff=1536,
+                  shared_ff=1536, ssm_state=128, ssm_groups=8,
+                  vocab=32000),
+    "medium": dict(width=4096, layers=2, heads=32, dim=128, rot_dim=64,
+                   vdim=128, kv_rank=512, experts=8, top=2, ff=3072,
+                   shared_ff=3072, ssm_state=128, ssm_groups=8,
+                   vocab=32000),
+}
+
+
+def _papunex_dir(s: dict, hybrid: bool) -> str:
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"]},
+           "router": {"experts": s["experts"], "top": s["top"],
+                      "scale": 1.0},
+           "shared": {"ff": s["shared_ff"]}}
+    att = {"type": "latent_attention",
+           "mixer": {"heads": s["heads"], "dim": s["dim"],
+                     "rot_dim": s["rot_dim"], "vdim": s["vdim"],
+                     "kv_rank": s["kv_rank"],
+                     "rot": {"base": 10000.0, "dims": s["rot_dim"]},
+                     "scale": (s["dim"] + s["rot_dim"]) ** -0.5},
+           "mlp": mlp}
+    ssm = {"type": "mamba2",
+           "mixer": {"heads": 2 * s["width"] // 64, "vdim": 64,
+                     "state": s["ssm_state"], "groups": s["ssm_groups"],
+                     "conv": 4, "norm_groups": s["ssm_groups"]},
+           "mlp": mlp}
+    layers = [ssm if hybrid and i % 2 else att
+              for i in range(s["layers"])]
+    cfg = {"architecture": "Papunex", "vocab": s["vocab"],
+           "width": s["width"], "embedding": {"scale": 1.0},
+           "norm": {"eps": 1e-5}, "logit_softcap": 30.0, "layers": layers}
+    d = tempfile.mkdtemp(prefix="papunex_bench_")
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return d
+
+
+def _deepseek_spec(s: dict):
+    from vllm_amd.config import ModelSpec
+
+    inter = s["ff"] * 2 // 3
+    return ModelSpec(
+        name="deepseek-like", architecture="deepseek",
+        vocab_size=s["vocab"], hidden_size=s["width"],
+        intermediate_size=inter, num_layers=s["layers"],
+        num_heads=s["heads"], num_kv_heads=s["heads"],
+        head_dim=s["dim"] + s["rot_dim"], rope_theta=10000.0,
+        max_position_embeddings=1 << 17, num_experts=s["experts"],
+        num_experts_per_tok=s["top"], moe_intermediate_size=inter,
+        num_shared_experts=1, first_dense_layers=0,
+        scoring_func="softmax", q_lora_rank=0, kv_lora_rank=s["kv_rank"],
+        qk_nope_head_dim=s["dim"], qk_rope_head_dim=s["rot_dim"],
+        v_head_dim=s["vdim"])
 
 
 def _gadilix_dir(s: dict) -> str:
@@ -85,6 +153,14 @@ def _engine(family: str, s: dict, max_len: int, batch: int, tokens: int):
     if family == "gadilix":
         mc = ModelConfig(model=_gadilix_dir(s), dtype="bf16",
                          max_model_len=max_len, load_format="dummy")
+    elif family in ("papunex", "papunex-hybrid"):
+        mc = ModelConfig(model=_papunex_dir(s, family.endswith("hybrid")),
+                         dtype="bf16", max_model_len=max_len,
+                         load_format="dummy")
+    elif family == "deepseek-like":
+        mc = ModelConfig(model="deepseek-like", dtype="bf16",
+                         max_model_len=max_len, load_format="dummy",
+                         spec=_deepseek_spec(s))
     else:
         mc = ModelConfig(model="mixtral-like", dtype="bf16",
                          max_model_len=max_len, load_format="dummy",
@@ -185,12 +261,20 @@ def _run(family: str, name: str, s: dict, prompt_len: int,
 def main(family: str, sizes: str, prompt_len: int = 4096,
          prefill_batch: int = 4, decode_batch: int = 64,
          decode_steps: int = 32, chunk_tokens: int = 8192) -> None:
-    if family != "gadilix":
-        raise SystemExit(f"unknown family {family!r} (known: gadilix)")
+    if family not in ("gadilix", "papunex"):
+        raise SystemExit(
+            f"unknown family {family!r} (known: gadilix, papunex)")
     if not torch.cuda.is_available():
         raise SystemExit("--compare-family needs a GPU")
+    table, fams = ((SIZES, ("gadilix", "mixtral-like"))
+                   if family == "gadilix" else
+                   (PAPUNEX_SIZES,
+                    ("papunex", "papunex-hybrid", "deepseek-like")))
+    only = os.environ.get("VLLM_AMD_COMPARE_ONLY")
+    if only:
+        fams = tuple(f for f in fams if f in only.split(","))
     for name in sizes.split(","):
-        s = SIZES[name]
-        for fam in ("gadilix", "mixtral-like"):
+        s = table[name]
+        for fam in fams:
             _run(fam, name, s, prompt_len, prefill_batch, decode_batch,
                  decode_steps, chunk_tokens)

@@ -244,14 +244,17 @@ _MOE_BM = 64  # must match moe::BM in csrc/moe.hip
 
 
 def _moe_hip_ok(hidden, w13, w2, activation):
-    if activation != "silu":
+    if activation not in ("silu", "relu2"):
         return False
     if hidden.dtype not in (torch.bfloat16, torch.float16):
         return False
     H = hidden.shape[1]
-    twoI = w13.shape[1]
+    n1 = w13.shape[1]
+    if activation == "relu2":
+        # Ungated: GEMM1 K=H%64, N=I%128; GEMM2 K=I%64, N=H%128.
+        return H % 128 == 0 and n1 % 128 == 0
     # GEMM1: K=H%64, N=2I%128; GEMM2: K=I%64, N=H%128.
-    return H % 128 == 0 and twoI % 128 == 0 and (twoI // 2) % 64 == 0
+    return H % 128 == 0 and n1 % 128 == 0 and (n1 // 2) % 64 == 0
 
 
 def moe_shuffle_weights(w):
@@ -266,15 +269,15 @@ def moe_shuffle_weights(w):
 
 
 def fused_moe_hip(hidden, w13, w2, topk_weights, topk_ids,
-                  w13_shuf=None, w2_shuf=None):
+                  w13_shuf=None, w2_shuf=None, activation="silu"):
     """Grouped-GEMM MFMA MoE (csrc/moe.hip): on-device token->expert
     sort into BM tiles, two MFMA GEMMs streaming each expert's weights,
     deterministic weighted combine. No host sync — hipGraph-capturable
     (role of the reference's fused_moe.py:299 + moe_align_sum_kernels.cu).
     """
     T, H = hidden.shape
-    E, twoI, _ = w13.shape
-    I = twoI // 2
+    E, twoI, _ = w13.shape      # ungated experts: the up width itself
+    I = w2.shape[2]
     k = topk_ids.shape[1]
     total = T * k
     dev = hidden.device
@@ -294,7 +297,7 @@ def fused_moe_hip(hidden, w13, w2, topk_weights, topk_ids,
                          twoI, H, k, total)
     else:
         _C.moe_gemm(hidden, w13, y, sorted_ids, expert_tiles, k, total)
-    act = silu_and_mul(y)
+    act = _C.relu2(y) if activation == "relu2" else silu_and_mul(y)
     y2 = torch.empty(em_max, H, dtype=hidden.dtype, device=dev)
     if w2_shuf is not None:
         _C.moe_gemm_shuf(act, w2_shuf, y2, sorted_ids, expert_tiles,
@@ -319,7 +322,8 @@ def fused_moe(hidden, w13, w2, topk_weights, topk_ids, activation="silu",
     """
     if _moe_hip_ok(hidden, w13, w2, activation):
         return fused_moe_hip(hidden, w13, w2, topk_weights, topk_ids,
-                             w13_shuf=w13_shuf, w2_shuf=w2_shuf)
+                             w13_shuf=w13_shuf, w2_shuf=w2_shuf,
+                             activation=activation)
     T, H = hidden.shape
     E = w13.shape[0]
     k = topk_ids.shape[1]

@@ -547,7 +547,19 @@ class ModelRunner:
                         dtype=self.dtype, device=self.device))
             if not self.layer_states:
                 self.layer_states = None
+            # Decode is captured when every routed layer's experts fit
+            # the grouped-GEMM kernels (the other expert path
+            # synchronizes with the host); state rows are staged into a
+            # static index buffer, padded entries use the scratch row.
             self.graph_runner = None
+            if (self.device.type == "cuda"
+                    and not self.config.model_config.enforce_eager
+                    and not self.config.model_config.lora_modules
+                    and self.pp_size == 1 and get_tp_world_size() == 1
+                    and self.dtype in (torch.bfloat16, torch.float16)
+                    and all(self._ungated_experts_capturable(e)
+                            for e in spec.layer_specs)):
+                self.graph_runner = DecodeGraphRunner(self)
             return
         if spec.layer_specs is not None:
             # One (k, v, pooled k, pooled v) tuple per layer RUN — layers
@@ -675,6 +687,16 @@ class ModelRunner:
             return True
         ff = int(ml["expert"]["ff"])
         return self.spec.hidden_size % 128 == 0 and ff % 64 == 0
+
+    def _ungated_experts_capturable(self, entry: dict) -> bool:
+        """Ungated (up -> act -> down) routed experts fit the
+        grouped-GEMM kernels (width % 128, ff % 128), or the layer
+        routes nothing."""
+        ml = entry.get("mlp")
+        if ml is None or ml.get("kind") != "moe":
+            return True
+        ff = int(ml["expert"]["ff"])
+        return self.spec.hidden_size % 128 == 0 and ff % 128 == 0
 
     def allocate_host_kv_pool(self, num_host_blocks: int) -> None:
         """Pinned host-RAM pool for offloaded prefix blocks: one tensor
