@@ -416,3 +416,60 @@ def test_greedy_generation_on_gpu(model_g):
             if float(top2[0] - top2[1]) > 1e-3:
                 assert tok == int(logits.argmax())
             seq.append(tok)
+
+
+def test_captured_decode_matches_eager(tmp_path):
+    """One-token steps replayed from captured hipGraphs (batch buckets
+    with padded rows, requests joining and leaving, state rows staged
+    per step, a context that passes 1024 keys) against the eager
+    engine: both run the same kernels, so they agree to rounding of
+    the library GEMMs' algorithm choice."""
+    layers = [
+        O.latent_entry(heads=4, dim=16, rot_dim=32, vdim=32, kv_rank=64,
+                       rot_dims=32, base=10000.0, mlp="moe", ff=128,
+                       experts=6, top=2, shared_ff=128),
+        O.mamba_entry(heads=4, vdim=32, state=24, groups=2, conv=4,
+                      norm_groups=2, mlp="dense", ff=128),
+        O.latent_entry(heads=8, dim=8, rot_dim=32, vdim=16, kv_rank=64,
+                       rot_dims=32, base=10000.0, kv_from=0, mlp=None),
+        O.latent_entry(heads=2, dim=8, rot_dim=6, vdim=12, kv_rank=20,
+                       rot_dims=6, mlp="moe", ff=128, experts=4, top=1,
+                       shared_ff=0),
+    ]
+    cfg = O.make_config(layers, vocab=80, width=128, embed_scale=3.0,
+                        softcap=25.0)
+    wt = O.random_weights(cfg, seed=5)
+    path = O.save_model(str(tmp_path / "m"), cfg, wt)
+    reqs = {"a": _tokens(1080, 80, 41), "b": _tokens(90, 80, 42),
+            "c": _tokens(70, 80, 43)}
+    steps = [([("a", reqs["a"][:1000], [999]),
+               ("b", reqs["b"][:50], [49])], [])]
+    for i in range(40):                       # two decode rows
+        steps.append(([("a", reqs["a"][1000 + i:1001 + i], [0]),
+                       ("b", reqs["b"][50 + i:51 + i], [0])],
+                      ["b"] if i == 39 else []))
+    steps.append(([("c", reqs["c"][:60], [59])], []))
+    for i in range(10):                       # other rows, other bucket
+        steps.append(([("a", reqs["a"][1040 + i:1041 + i], [0]),
+                       ("c", reqs["c"][60 + i:61 + i], [0])],
+                      ["a", "c"] if i == 9 else []))
+    for i in range(30):                       # one row alone
+        steps.append(([("d", _tokens(1, 80, 100 + i), [0])],
+                      ["d"] if i == 29 else []))
+    graph, core = run_schedule(path, steps, dtype="bfloat16",
+                               max_tokens=1408, device=DEV,
+                               enforce_eager=False)
+    assert core.worker.runner.graph_runner is not None
+    assert core.worker.runner.graph_runner.graphs, "nothing was captured"
+    eager, _ = run_schedule(path, steps, dtype="bfloat16", max_tokens=1408,
+                            device=DEV)
+    assert graph.keys() == eager.keys()
+    errs = []
+    for key, got in graph.items():
+        d = got - eager[key]
+        d = d - d.mean()
+        scale = (eager[key] - eager[key].mean()).pow(2).mean().sqrt().item()
+        errs.append(d.pow(2).mean().sqrt().item() / max(scale, 1e-3))
+    errs.sort()
+    assert errs[len(errs) // 2] <= 0.02, errs[len(errs) // 2]
+    assert errs[int(0.95 * len(errs))] <= 0.1, errs[-10:]
