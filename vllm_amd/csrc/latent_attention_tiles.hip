@@ -16,7 +16,8 @@
 //            (m = sink_h, l = 1) when the layer has a sink.
 //   PV : wave w owns value columns [w*LORA/4, (w+1)*LORA/4).
 // The subtile is staged once: [tok][DK] (swizzled, QK reads rows) plus a
-// transposed copy of the first LORA columns [col][tok] (PV reads rows).
+// transposed copy of the first LORA columns [col][token pair] (PV reads
+// rows), written without LDS bank conflicts.
 
 #include <torch/all.h>
 #include <c10/hip/HIPStream.h>
@@ -34,6 +35,7 @@ constexpr int PART = 1024;       // tokens per decode partition
 constexpr int THREADS = 256;
 constexpr float NEG_INF = -1e30f;
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr int VS = 18;           // dwords per column of the transposed V
 
 DEVINL int swz(int row, int byte_off) { return byte_off ^ ((row & 7) << 4); }
 
@@ -109,7 +111,7 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
   const int t_end = single ? vis_end : min(t_begin + PART, vis_end);
 
   __shared__ short k_lds[SUB * KROW / 2];  // [tok][DK], 16 B slots
-  __shared__ short vt_lds[LORA * SUB];    // [col][tok]
+  __shared__ uint32_t vt_lds[LORA * VS];  // [col][token pair]
   __shared__ short p_lds[HG * SUB];       // [row][tok] bf16
   __shared__ float m_st[HG], l_st[HG], f_st[HG];
   __shared__ float wmax[2][HG], wsum[2][HG];
@@ -184,23 +186,38 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
   const int* bt = block_table + (long)grp.req * bt_stride;
 
   for (int sub0 = t_begin; sub0 < t_end; sub0 += SUB) {
-    // ---- stage 32 cached rows.
-    for (int c = tid; c < SUB * (DK / 8); c += THREADS) {
-      const int tok = c / (DK / 8);
-      const int f8 = c % (DK / 8);
-      const int t_glob = sub0 + tok;
-      s16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    // ---- stage 32 cached rows. A thread takes one 16 B column chunk of
+    // a PAIR of adjacent tokens: the pair's values go into the
+    // transposed copy as one dword per column, and with token pairs
+    // fastest across lanes and a column stride of VS = 18 dwords a
+    // wave's 64 stores fall on 64 different banks.
+    for (int c = tid; c < (SUB / 2) * (DK / 8); c += THREADS) {
+      const int tp = c % (SUB / 2);
+      const int f8 = c / (SUB / 2);
+      const int t_glob = sub0 + 2 * tp;
+      s16x8 v0 = {0, 0, 0, 0, 0, 0, 0, 0};
+      s16x8 v1 = {0, 0, 0, 0, 0, 0, 0, 0};
       if (t_glob < t_end) {
         const int blk = bt[t_glob / block_size];
-        v = *reinterpret_cast<const s16x8*>(
+        v0 = *reinterpret_cast<const s16x8*>(
             kv + ((long)blk * block_size + t_glob % block_size) * DK +
             f8 * 8);
       }
+      if (t_glob + 1 < t_end) {
+        const int blk = bt[(t_glob + 1) / block_size];
+        v1 = *reinterpret_cast<const s16x8*>(
+            kv + ((long)blk * block_size + (t_glob + 1) % block_size) * DK +
+            f8 * 8);
+      }
       *reinterpret_cast<s16x8*>(reinterpret_cast<char*>(k_lds) +
-                                kaddr(tok, f8 * 16)) = v;
+                                kaddr(2 * tp, f8 * 16)) = v0;
+      *reinterpret_cast<s16x8*>(reinterpret_cast<char*>(k_lds) +
+                                kaddr(2 * tp + 1, f8 * 16)) = v1;
       if (f8 * 8 < LORA) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) vt_lds[(f8 * 8 + j) * SUB + tok] = v[j];
+        for (int j = 0; j < 8; ++j)
+          vt_lds[(f8 * 8 + j) * VS + tp] =
+              (uint32_t)(uint16_t)v0[j] | ((uint32_t)(uint16_t)v1[j] << 16);
       }
     }
     __syncthreads();
@@ -286,8 +303,13 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
 #pragma unroll
       for (int nf = 0; nf < NF; ++nf) {
         const int col = wave * WC + nf * 16 + l16;
-        s16x8 bfrag =
-            *reinterpret_cast<const s16x8*>(vt_lds + col * SUB + l4 * 8);
+        // 8 tokens = 4 dwords; columns are 8 B aligned (VS is even).
+        const uint32_t* vp = vt_lds + col * VS + l4 * 4;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vp);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vp + 2);
+        union { uint32_t u[4]; s16x8 v; } pk;
+        pk.u[0] = lo.x; pk.u[1] = lo.y; pk.u[2] = hi.x; pk.u[3] = hi.y;
+        s16x8 bfrag = pk.v;
         o_acc[mt][nf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
             afrag, bfrag, o_acc[mt][nf], 0, 0, 0);
       }

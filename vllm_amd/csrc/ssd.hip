@@ -45,6 +45,73 @@ DEVINL int sfind_req(const int* __restrict__ qsl, int num_reqs, int t) {
   return lo;
 }
 
+// Sum over the 16 lanes of a DPP row (rotations by 8, 4, 2, 1); every
+// lane ends with the total.
+DEVINL float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+
+// Four taps, 16-bit input, eight channels per thread with 16 B loads;
+// output fp32 (TO = F32Tag) or the input type.
+template <typename T, typename TO>
+__global__ __launch_bounds__(SB) void causal_conv4_silu_vec_kernel(
+    typename ET<TO>::t* __restrict__ out,              // [T, C]
+    const short* __restrict__ x, const int64_t x_st,
+    const short* __restrict__ w,                       // [C, 4]
+    const short* __restrict__ bias,                    // [C]
+    const short* __restrict__ conv_state,              // [rows, C, 3]
+    const int64_t* __restrict__ state_rows, const int* __restrict__ qsl,
+    const int num_reqs, const int C) {
+  constexpr int K = 4;
+  const int ch0 = (blockIdx.y * SB + threadIdx.x) * 8;
+  const int t = blockIdx.x;
+  if (ch0 >= C) return;
+  const int r = sfind_req(qsl, num_reqs, t);
+  const int s = qsl[r];
+  const short* hist =
+      conv_state == nullptr
+          ? nullptr
+          : conv_state + (state_rows[r] * C + ch0) * (int64_t)(K - 1);
+  // w for channel e, tap j sits at wv[(e * 4 + j) / 8][(e * 4 + j) % 8].
+  s16x8 wv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    wv[i] = *reinterpret_cast<const s16x8*>(w + (int64_t)ch0 * K + i * 8);
+  const s16x8 bv = *reinterpret_cast<const s16x8*>(bias + ch0);
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = ET<T>::ld(bv[e]);
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const int src = t - (K - 1) + j;
+    if (src >= s) {
+      const s16x8 xv =
+          *reinterpret_cast<const s16x8*>(x + (int64_t)src * x_st + ch0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        acc[e] += ET<T>::ld(wv[(e * 4 + j) / 8][(e * 4 + j) % 8]) *
+                  ET<T>::ld(xv[e]);
+    } else if (hist != nullptr) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        acc[e] += ET<T>::ld(wv[(e * 4 + j) / 8][(e * 4 + j) % 8]) *
+                  ET<T>::ld(hist[e * (K - 1) + (K - 1) + (src - s)]);
+    }
+  }
+  typename ET<TO>::t* o = out + (int64_t)t * C + ch0;
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    o[e] = ET<TO>::st(acc[e] / (1.f + expf(-acc[e])));
+}
+
 template <typename T, typename TO>
 __global__ __launch_bounds__(SB) void causal_conv_silu_kernel(
     typename ET<TO>::t* __restrict__ out,              // [T, C]
@@ -184,9 +251,7 @@ __global__ __launch_bounds__(SB) void ssd_scan_kernel(
       }
 #pragma unroll
       for (int a = 0; a < PA; ++a) {
-        float v = yacc[a];
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+        const float v = row16_sum(yacc[a]);
         if (sl == 0) ys[tt][pl + 16 * a] = v;
       }
     }
@@ -280,6 +345,29 @@ torch::Tensor causal_conv_silu(torch::Tensor x, torch::Tensor weight,
   auto out = torch::empty({T, C}, x.options().dtype(out_dtype));
   if (T == 0) return out;
   auto stream = c10::hip::getCurrentHIPStream().stream();
+  const bool vec4 = K == 4 && C % 8 == 0 && x.stride(0) % 8 == 0 &&
+                    x.storage_offset() % 8 == 0 &&
+                    x.scalar_type() != torch::kFloat32;
+  if (vec4) {
+    const dim3 gv(T, (C / 8 + SB - 1) / SB);
+#define LV2(TT, TO)                                                        \
+  hipLaunchKernelGGL(                                                      \
+      (causal_conv4_silu_vec_kernel<TT, TO>), gv, dim3(SB), 0, stream,     \
+      (ET<TO>::t*)out.data_ptr(), (const short*)x.data_ptr(), x.stride(0), \
+      (const short*)weight.data_ptr(), (const short*)bias.data_ptr(),      \
+      has_state ? (const short*)conv_state->data_ptr() : nullptr,          \
+      has_state ? state_rows->data_ptr<int64_t>() : nullptr,               \
+      query_start_loc.data_ptr<int>(), num_reqs, C)
+    if (x.scalar_type() == torch::kBFloat16) {
+      if (out_dtype == torch::kFloat32) { LV2(BF16Tag, F32Tag); }
+      else { LV2(BF16Tag, BF16Tag); }
+    } else {
+      if (out_dtype == torch::kFloat32) { LV2(FP16Tag, F32Tag); }
+      else { LV2(FP16Tag, FP16Tag); }
+    }
+#undef LV2
+    HIP_CHECK_KERNEL();
+  }
   const dim3 grid(T, (C + SB - 1) / SB);
 #define L2(TT, TO)                                                         \
   hipLaunchKernelGGL(                                                      \
@@ -292,7 +380,7 @@ torch::Tensor causal_conv_silu(torch::Tensor x, torch::Tensor weight,
       query_start_loc.data_ptr<int>(), num_reqs, C, K)
 #define L1(TT)                                                             \
   if (out_dtype == torch::kFloat32) { L2(TT, F32Tag); } else { L2(TT, TT); }
-  SDISPATCH(x.scalar_type(), L1);
+  if (!vec4) { SDISPATCH(x.scalar_type(), L1); }
 #undef L1
 #undef L2
   HIP_CHECK_KERNEL();
@@ -347,7 +435,13 @@ torch::Tensor ssd_scan(torch::Tensor xbc, int64_t heads, int64_t head_dim,
   auto stream = c10::hip::getCurrentHIPStream().stream();
   // Columns per workgroup 16*PA with PA in {1,2,4}; wider heads take
   // several slabs (columns are independent). NK covers N in 16s.
-  const int pa = P <= 16 ? 1 : (P <= 32 ? 2 : 4);
+  // Fewer columns per workgroup when the batch alone cannot fill the
+  // chip (a few long prompts): the recurrence is sequential in time, so
+  // width is the only parallelism there is.
+  int pa = P <= 16 ? 1 : (P <= 32 ? 2 : 4);
+  while (pa > 1 &&
+         (int64_t)num_reqs * Hm * ((P + 16 * pa - 1) / (16 * pa)) < 1024)
+    pa /= 2;
   const int nk_need = (N + 15) / 16;
   const int nk = nk_need <= 2 ? 2 : (nk_need <= 4 ? 4 : (nk_need <= 8 ? 8
                                                                       : 16));
