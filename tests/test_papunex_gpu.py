@@ -140,7 +140,7 @@ def test_latent_attention_tiles_bf16(L, R, H):
     tokens per workgroup (H < 32), several workgroups per token
     (H > 32), with a sink."""
     torch.manual_seed(L + R + H)
-    T = 140 if H > 8 else 1200     # few heads: also past 1024 keys
+    T = 140 if H > 8 else 1200     # few heads: also a long context
     q_abs = (torch.randn(T, H, L) * (3.0 / math.sqrt(L))).bfloat16().float()
     q_rot = torch.randn(T, H, R).bfloat16().float()
     rows = torch.randn(T, L + R).bfloat16().float()
@@ -155,8 +155,8 @@ def test_latent_attention_tiles_bf16(L, R, H):
 
 
 def test_latent_attention_batch_of_decodes_and_portions():
-    """Decode rows of unequal context (one past 1024 keys: two key
-    partitions) beside two prompt portions, shuffled pages."""
+    """Decode rows of unequal context (one to five key partitions)
+    beside two prompt portions, shuffled pages."""
     from vllm_amd import ops
 
     torch.manual_seed(4)
@@ -224,15 +224,17 @@ def test_conv_kernel(K, dtype):
     assert got.dtype == dtype
 
 
+@pytest.mark.parametrize("lens", [[1, 1, 70, 33, 2], [1, 700, 256, 2, 257]])
 @pytest.mark.parametrize("Hm,P,G,N", [(8, 32, 2, 48), (4, 64, 1, 128),
                                       (3, 5, 3, 3), (2, 100, 1, 200),
                                       (6, 16, 2, 17)])
-def test_scan_kernel(Hm, P, G, N):
+def test_scan_kernel(Hm, P, G, N, lens):
+    """Short portions run sequentially; a portion longer than 256 tokens
+    switches the whole batch to parallel segments with a carry pass."""
     from vllm_amd import ops
 
     torch.manual_seed(Hm * P)
     R = _ref_ops()
-    lens = [1, 1, 70, 33, 2]
     T = sum(lens)
     xbc = torch.randn(T, Hm * P + 2 * G * N)
     dt = torch.randn(T, Hm + 4)
@@ -248,9 +250,9 @@ def test_scan_kernel(Hm, P, G, N):
     got = ops.ssd_scan(xbc.to(DEV), Hm, P, G, N,
                        dt.to(DEV)[:, 2:2 + Hm], dt_bias.to(DEV),
                        a_log.to(DEV), d_skip.to(DEV), st, rows.to(DEV),
-                       qsl.to(DEV))
-    _close(got, ref, 2e-5)
-    _close(st, st_ref, 2e-5)
+                       qsl.to(DEV), max_query_len=max(lens))
+    _close(got, ref, 5e-5)
+    _close(st, st_ref, 5e-5)
     got = ops.ssd_scan(xbc.to(DEV), Hm, P, G, N,
                        dt.to(DEV)[:, 2:2 + Hm].bfloat16(), dt_bias.to(DEV),
                        a_log.to(DEV), d_skip.to(DEV), None, None,
@@ -421,7 +423,7 @@ def test_greedy_generation_on_gpu(model_g):
 def test_captured_decode_matches_eager(tmp_path):
     """One-token steps replayed from captured hipGraphs (batch buckets
     with padded rows, requests joining and leaving, state rows staged
-    per step, a context that passes 1024 keys) against the eager
+    per step, a context of several key partitions) against the eager
     engine: both run the same kernels, so they agree to rounding of
     the library GEMMs' algorithm choice."""
     layers = [

@@ -138,7 +138,8 @@ torch::Tensor ssd_scan(torch::Tensor xbc, int64_t heads, int64_t head_dim,
                        torch::Tensor d_skip,
                        c10::optional<torch::Tensor> ssm_state,
                        c10::optional<torch::Tensor> state_rows,
-                       torch::Tensor query_start_loc);
+                       torch::Tensor query_start_loc,
+                       int64_t max_query_len);
 torch::Tensor gated_group_rms_norm(torch::Tensor y, torch::Tensor z,
                                    torch::Tensor weight, double eps,
                                    int64_t groups,
@@ -248,7 +249,7 @@ TORCH_LIBRARY(vllm_amd, m) {
   m.def("ssd_scan(Tensor xbc, int heads, int head_dim, int groups, "
         "int state, Tensor dt, Tensor dt_bias, Tensor a_log, "
         "Tensor d_skip, Tensor(a!)? ssm_state, Tensor? state_rows, "
-        "Tensor query_start_loc) -> Tensor");
+        "Tensor query_start_loc, int max_query_len) -> Tensor");
   m.def("gated_group_rms_norm(Tensor y, Tensor z, Tensor weight, "
         "float eps, int groups, ScalarType out_dtype) -> Tensor");
   // Custom xGMI collectives (comms.hip). init/connect/destroy are

@@ -9,7 +9,7 @@
 // walks the keys 0 .. last visible in 32-token subtiles. Each row is
 // masked to its own position (causal), so prefill chunks and decode
 // rows run the same code; decode batches additionally split the keys
-// into 1024-token partitions merged by latent_tile_reduce_kernel.
+// into 256-token partitions merged by latent_tile_reduce_kernel.
 //   QK : wave (mtile = w&1, ntile = w>>1) computes a 16 x 16 score tile.
 //   softmax: online, fp32, log2 domain; per-row max/sum shared through
 //            LDS. The running state of partition 0 starts at
@@ -31,7 +31,7 @@ namespace lat {
 
 constexpr int HG = 32;           // rows per workgroup
 constexpr int SUB = 32;          // cached tokens per subtile
-constexpr int PART = 1024;       // tokens per decode partition
+constexpr int PART = 256;        // tokens per decode partition
 constexpr int THREADS = 256;
 constexpr float NEG_INF = -1e30f;
 constexpr float LOG2E = 1.4426950408889634f;

@@ -165,6 +165,59 @@ __global__ __launch_bounds__(SB) void conv_state_update_kernel(
   }
 }
 
+// A long prompt portion is cut into segments of SSD_SEG tokens that run
+// side by side: pass 1 runs every segment from a zero state and keeps
+// its end state and the product of its decays, ssd_seg_carry_kernel
+// chains those per request (S_in of segment j+1 = decay_j S_in_j + end_j)
+// and leaves each segment's true start state in the same buffer, pass 3
+// reruns the segments from there and writes y.
+constexpr int SSD_SEG = 256;
+constexpr int MODE_WHOLE = 0, MODE_LOCAL = 1, MODE_FINAL = 3;
+
+struct Seg {
+  int req, t0, t1;
+};
+
+DEVINL Seg find_seg(int g, const int* __restrict__ qsl, int num_reqs) {
+  for (int r = 0; r < num_reqs; ++r) {
+    const int n = qsl[r + 1] - qsl[r];
+    const int segs = (n + SSD_SEG - 1) / SSD_SEG;
+    if (g < segs) {
+      const int t0 = qsl[r] + g * SSD_SEG;
+      return Seg{r, t0, min(t0 + SSD_SEG, qsl[r + 1])};
+    }
+    g -= segs;
+  }
+  return Seg{-1, 0, 0};
+}
+
+__global__ __launch_bounds__(SB) void ssd_seg_carry_kernel(
+    float* __restrict__ seg_state,         // [segs, Hm, P*N]
+    const float* __restrict__ seg_decay,   // [segs, Hm]
+    float* __restrict__ ssm_state,         // [rows, Hm, P*N] or null
+    const int64_t* __restrict__ state_rows, const int* __restrict__ qsl,
+    const int Hm, const int PN) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int i = blockIdx.z * SB + threadIdx.x;
+  if (i >= PN) return;
+  int g0 = 0;
+  for (int q = 0; q < r; ++q)
+    g0 += (qsl[q + 1] - qsl[q] + SSD_SEG - 1) / SSD_SEG;
+  const int nseg = (qsl[r + 1] - qsl[r] + SSD_SEG - 1) / SSD_SEG;
+  if (nseg == 0) return;
+  float* st = ssm_state == nullptr
+                  ? nullptr
+                  : ssm_state + (state_rows[r] * Hm + h) * (int64_t)PN + i;
+  float carry = st != nullptr ? *st : 0.f;
+  for (int j = 0; j < nseg; ++j) {
+    float* slot = seg_state + ((int64_t)(g0 + j) * Hm + h) * PN + i;
+    const float end = *slot;
+    *slot = carry;
+    carry = seg_decay[(int64_t)(g0 + j) * Hm + h] * carry + end;
+  }
+  if (st != nullptr) *st = carry;
+}
+
 template <int PA, int NK>
 __global__ __launch_bounds__(SB) void ssd_scan_kernel(
     float* __restrict__ y,                 // [T, Hm, P]
@@ -175,17 +228,27 @@ __global__ __launch_bounds__(SB) void ssd_scan_kernel(
     const float* __restrict__ d_skip,
     float* __restrict__ ssm_state,         // [rows, Hm, P, N] or null
     const int64_t* __restrict__ state_rows, const int* __restrict__ qsl,
-    const int Hm, const int P) {
+    const int Hm, const int P, const int mode, const int num_reqs,
+    float* __restrict__ seg_state, float* __restrict__ seg_decay) {
   __shared__ float Bs[SSD_TT][SSD_MAX_N];
   __shared__ float Cs[SSD_TT][SSD_MAX_N];
   __shared__ float xs[SSD_TT][16 * PA];
   __shared__ float ys[SSD_TT][16 * PA];
   __shared__ float dts[SSD_TT], dec[SSD_TT];
 
-  const int r = blockIdx.x, h = blockIdx.y;
+  const int h = blockIdx.y;
   const int p0 = blockIdx.z * 16 * PA;
-  const int s = qsl[r], e = qsl[r + 1];
-  if (s >= e) return;
+  int r = blockIdx.x, s, e;
+  if (mode == MODE_WHOLE) {
+    s = qsl[r];
+    e = qsl[r + 1];
+  } else {
+    const Seg sg = find_seg(blockIdx.x, qsl, num_reqs);
+    r = sg.req;
+    s = sg.t0;
+    e = sg.t1;
+  }
+  if (r < 0 || s >= e) return;
   const int g = h / (Hm / G);
   const int tid = threadIdx.x;
   const int sl = tid & 15, pl = tid >> 4;
@@ -193,19 +256,25 @@ __global__ __launch_bounds__(SB) void ssd_scan_kernel(
   const float bias = dt_bias[h], dsk = d_skip[h];
 
   float S[PA][NK];
-  float* st = ssm_state == nullptr
-                  ? nullptr
-                  : ssm_state + (state_rows[r] * Hm + h) * (int64_t)P * N;
+  float* st;
+  if (mode == MODE_WHOLE)
+    st = ssm_state == nullptr
+             ? nullptr
+             : ssm_state + (state_rows[r] * Hm + h) * (int64_t)P * N;
+  else
+    st = seg_state + ((int64_t)blockIdx.x * Hm + h) * (int64_t)P * N;
+  const bool load_state = st != nullptr && mode != MODE_LOCAL;
 #pragma unroll
   for (int a = 0; a < PA; ++a) {
     const int p = p0 + pl + 16 * a;
 #pragma unroll
     for (int k = 0; k < NK; ++k) {
       const int n = sl + 16 * k;
-      S[a][k] = (st != nullptr && p < P && n < N) ? st[(int64_t)p * N + n]
-                                                  : 0.f;
+      S[a][k] = (load_state && p < P && n < N) ? st[(int64_t)p * N + n]
+                                               : 0.f;
     }
   }
+  float dprod = 1.f;
 
   const float* Bg = xbc + inner + g * N;
   const float* Cg = xbc + inner + G * N + g * N;
@@ -232,6 +301,7 @@ __global__ __launch_bounds__(SB) void ssd_scan_kernel(
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
       const float dtp = dts[tt], dc = dec[tt];
+      dprod *= dc;
       float xp[PA], yacc[PA];
 #pragma unroll
       for (int a = 0; a < PA; ++a) {
@@ -256,14 +326,18 @@ __global__ __launch_bounds__(SB) void ssd_scan_kernel(
       }
     }
     __syncthreads();
-    for (int i = tid; i < nt * 16 * PA; i += SB) {
-      const int tt = i / (16 * PA), pp = i - tt * (16 * PA);
-      if (p0 + pp < P)
-        y[((int64_t)(t0 + tt) * Hm + h) * P + p0 + pp] =
-            ys[tt][pp] + dsk * xs[tt][pp];
+    if (mode != MODE_LOCAL) {
+      for (int i = tid; i < nt * 16 * PA; i += SB) {
+        const int tt = i / (16 * PA), pp = i - tt * (16 * PA);
+        if (p0 + pp < P)
+          y[((int64_t)(t0 + tt) * Hm + h) * P + p0 + pp] =
+              ys[tt][pp] + dsk * xs[tt][pp];
+      }
     }
   }
-  if (st != nullptr) {
+  if (mode == MODE_LOCAL && blockIdx.z == 0 && tid == 0)
+    seg_decay[(int64_t)blockIdx.x * Hm + h] = dprod;
+  if (st != nullptr && mode != MODE_FINAL) {
 #pragma unroll
     for (int a = 0; a < PA; ++a) {
       const int p = p0 + pl + 16 * a;
@@ -405,7 +479,8 @@ torch::Tensor ssd_scan(torch::Tensor xbc, int64_t heads, int64_t head_dim,
                        torch::Tensor d_skip,
                        c10::optional<torch::Tensor> ssm_state,
                        c10::optional<torch::Tensor> state_rows,
-                       torch::Tensor query_start_loc) {
+                       torch::Tensor query_start_loc,
+                       int64_t max_query_len) {
   const int Hm = heads, P = head_dim, G = groups, N = state;
   TORCH_CHECK(xbc.dim() == 2 && xbc.is_contiguous() &&
               xbc.scalar_type() == torch::kFloat32);
@@ -438,27 +513,54 @@ torch::Tensor ssd_scan(torch::Tensor xbc, int64_t heads, int64_t head_dim,
   // Fewer columns per workgroup when the batch alone cannot fill the
   // chip (a few long prompts): the recurrence is sequential in time, so
   // width is the only parallelism there is.
+  const bool segmented = max_query_len > SSD_SEG;
+  const int nseg = segmented ? (T + SSD_SEG - 1) / SSD_SEG + num_reqs : 0;
+  const int gx = segmented ? nseg : num_reqs;
+  torch::Tensor seg_state, seg_decay;
+  if (segmented) {
+    seg_state = torch::empty({(int64_t)nseg * Hm * P * N}, xbc.options());
+    seg_decay = torch::empty({(int64_t)nseg * Hm}, xbc.options());
+  }
   int pa = P <= 16 ? 1 : (P <= 32 ? 2 : 4);
   while (pa > 1 &&
-         (int64_t)num_reqs * Hm * ((P + 16 * pa - 1) / (16 * pa)) < 1024)
+         (int64_t)gx * Hm * ((P + 16 * pa - 1) / (16 * pa)) < 1024)
     pa /= 2;
   const int nk_need = (N + 15) / 16;
   const int nk = nk_need <= 2 ? 2 : (nk_need <= 4 ? 4 : (nk_need <= 8 ? 8
                                                                       : 16));
-  const dim3 grid(num_reqs, Hm, (P + 16 * pa - 1) / (16 * pa));
-#define L2(PA_, NK_)                                                       \
+  const dim3 grid(gx, Hm, (P + 16 * pa - 1) / (16 * pa));
+  float* st_ptr =
+      ssm_state.has_value() ? ssm_state->data_ptr<float>() : nullptr;
+  const int64_t* rows_ptr =
+      ssm_state.has_value() ? state_rows->data_ptr<int64_t>() : nullptr;
+#define L2(PA_, NK_, MODE_)                                                \
   hipLaunchKernelGGL(                                                      \
       (ssd_scan_kernel<PA_, NK_>), grid, dim3(SB), 0, stream,              \
       y.data_ptr<float>(), xbc.data_ptr<float>(), Cc, Hm * P, G, N,        \
       dt.data_ptr<float>(), dt.stride(0), dt_bias.data_ptr<float>(),       \
-      a_log.data_ptr<float>(), d_skip.data_ptr<float>(),                   \
-      ssm_state.has_value() ? ssm_state->data_ptr<float>() : nullptr,      \
-      ssm_state.has_value() ? state_rows->data_ptr<int64_t>() : nullptr,   \
-      query_start_loc.data_ptr<int>(), Hm, P)
-#define L1(PA_)                                                            \
-  if (nk == 2) { L2(PA_, 2); } else if (nk == 4) { L2(PA_, 4); }           \
-  else if (nk == 8) { L2(PA_, 8); } else { L2(PA_, 16); }
-  if (pa == 1) { L1(1); } else if (pa == 2) { L1(2); } else { L1(4); }
+      a_log.data_ptr<float>(), d_skip.data_ptr<float>(), st_ptr, rows_ptr, \
+      query_start_loc.data_ptr<int>(), Hm, P, MODE_, num_reqs,             \
+      segmented ? seg_state.data_ptr<float>() : nullptr,                   \
+      segmented ? seg_decay.data_ptr<float>() : nullptr)
+#define L1(PA_, MODE_)                                                     \
+  if (nk == 2) { L2(PA_, 2, MODE_); } else if (nk == 4) { L2(PA_, 4, MODE_); } \
+  else if (nk == 8) { L2(PA_, 8, MODE_); } else { L2(PA_, 16, MODE_); }
+#define L0(MODE_)                                                          \
+  if (pa == 1) { L1(1, MODE_); } else if (pa == 2) { L1(2, MODE_); }       \
+  else { L1(4, MODE_); }
+  if (!segmented) {
+    L0(MODE_WHOLE);
+  } else {
+    L0(MODE_LOCAL);
+    const int PN = P * N;
+    hipLaunchKernelGGL(ssd_seg_carry_kernel,
+                       dim3(num_reqs, Hm, (PN + SB - 1) / SB), dim3(SB), 0,
+                       stream, seg_state.data_ptr<float>(),
+                       seg_decay.data_ptr<float>(), st_ptr, rows_ptr,
+                       query_start_loc.data_ptr<int>(), Hm, PN);
+    L0(MODE_FINAL);
+  }
+#undef L0
 #undef L1
 #undef L2
   HIP_CHECK_KERNEL();

@@ -88,7 +88,8 @@ class Mamba2Mixer(nn.Module):
             out_dtype=torch.float32)
         y = ops.ssd_scan(xbc, self.heads, self.head_dim, self.groups,
                          self.state, dt, self.dt_bias, self.A_log, self.D,
-                         ssm_state, meta.state_rows, meta.query_start_loc)
+                         ssm_state, meta.state_rows, meta.query_start_loc,
+                         max_query_len=meta.max_query_len)
         y = ops.gated_group_rms_norm(
             y.view(T, self.inner), z, self.norm_weight, self.eps,
             self.norm_groups, h.dtype)

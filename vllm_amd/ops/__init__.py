@@ -284,10 +284,16 @@ def causal_conv_silu(x, weight, bias, conv_state, state_rows,
 
 
 def ssd_scan(xbc, heads, head_dim, groups, state, dt, dt_bias, a_log,
-             d_skip, ssm_state, state_rows, query_start_loc):
-    return get_backend(xbc.device).ssd_scan(
+             d_skip, ssm_state, state_rows, query_start_loc,
+             max_query_len=0):
+    backend = get_backend(xbc.device)
+    if backend is _torch_ref:
+        return backend.ssd_scan(
+            xbc, heads, head_dim, groups, state, dt, dt_bias, a_log,
+            d_skip, ssm_state, state_rows, query_start_loc)
+    return backend.ssd_scan(
         xbc, heads, head_dim, groups, state, dt, dt_bias, a_log, d_skip,
-        ssm_state, state_rows, query_start_loc)
+        ssm_state, state_rows, query_start_loc, max_query_len)
 
 
 def gated_group_rms_norm(y, z, weight, eps, groups, out_dtype):

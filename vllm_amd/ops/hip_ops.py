@@ -516,11 +516,15 @@ def causal_conv_silu(x, weight, bias, conv_state, state_rows,
 
 
 def ssd_scan(xbc, heads, head_dim, groups, state, dt, dt_bias, a_log,
-             d_skip, ssm_state, state_rows, query_start_loc):
+             d_skip, ssm_state, state_rows, query_start_loc,
+             max_query_len=0):
+    """max_query_len (a host-side bound on the longest portion) lets
+    long portions run as parallel segments; 0 = unknown, sequential."""
     return _C.ssd_scan(
         xbc, heads, head_dim, groups, state, dt.float(), dt_bias, a_log,
         d_skip, ssm_state,
-        state_rows if ssm_state is not None else None, query_start_loc)
+        state_rows if ssm_state is not None else None, query_start_loc,
+        max_query_len)
 
 
 def gated_group_rms_norm(y, z, weight, eps, groups, out_dtype):
