@@ -535,3 +535,40 @@ def test_greedy_generation_through_llm(model_a):
             if float(top2[0] - top2[1]) > 1e-3:
                 assert tok == int(logits.argmax())
             seq.append(tok)
+
+
+def test_served_over_http(model_a):
+    """The OpenAI-compatible server loads the folder like any other
+    model; token-id prompt, greedy completion, the oracle's tokens (the
+    family has no tokenizer: ids come back as text bytes)."""
+    from fastapi.testclient import TestClient
+
+    from vllm_amd.engine.arg_utils import EngineArgs
+    from vllm_amd.entrypoints.openai.api_server import make_server
+
+    path, cfg, wt = model_a
+    prompt = _tokens(9, cfg["vocab"], 77)
+    seq = list(prompt)
+    sure = True
+    for _ in range(4):
+        logits = O.forward(cfg, wt, seq)[-1]
+        top2 = logits.topk(2).values
+        sure = sure and float(top2[0] - top2[1]) > 1e-3
+        seq.append(int(logits.argmax()))
+    args = EngineArgs(model=path, model_path=path, load_format="safetensors",
+                      dtype="fp32", device="cpu", num_gpu_blocks=8,
+                      max_model_len=256, max_num_seqs=4,
+                      max_num_batched_tokens=64)
+    app, state = make_server(args, None)
+    try:
+        with TestClient(app) as c:
+            r = c.post("/v1/completions", json={
+                "model": path, "prompt": prompt, "max_tokens": 4,
+                "temperature": 0})
+            assert r.status_code == 200, r.text
+    finally:
+        state.engine.shutdown()
+    text = r.json()["choices"][0]["text"]
+    assert len(text) == 4
+    if sure:
+        assert [ord(ch) for ch in text] == seq[len(prompt):]
