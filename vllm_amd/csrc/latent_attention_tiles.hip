@@ -9,13 +9,13 @@
 // walks the keys 0 .. last visible in 32-token subtiles. Each row is
 // masked to its own position (causal), so prefill chunks and decode
 // rows run the same code; decode batches additionally split the keys
-// into 256-token partitions merged by latent_tile_reduce_kernel.
+// into 1024-token partitions merged by latent_tile_reduce_kernel.
 //   QK : wave (mtile = w&1, ntile = w>>1) computes a 16 x 16 score tile.
 //   softmax: online, fp32, log2 domain; per-row max/sum shared through
 //            LDS. The running state of partition 0 starts at
 //            (m = sink_h, l = 1) when the layer has a sink.
 //   PV : wave w owns value columns [w*LORA/4, (w+1)*LORA/4).
-// The subtile is staged once: [tok][DK] (swizzled, QK reads rows) plus a
+// The subtile is staged once: [tok][DK] (padded rows, QK reads rows) plus a
 // transposed copy of the first LORA columns [col][token pair] (PV reads
 // rows), written without LDS bank conflicts.
 
@@ -31,13 +31,11 @@ namespace lat {
 
 constexpr int HG = 32;           // rows per workgroup
 constexpr int SUB = 32;          // cached tokens per subtile
-constexpr int PART = 256;        // tokens per decode partition
+constexpr int PART = 1024;       // tokens per decode partition
 constexpr int THREADS = 256;
 constexpr float NEG_INF = -1e30f;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int VS = 18;           // dwords per column of the transposed V
-
-DEVINL int swz(int row, int byte_off) { return byte_off ^ ((row & 7) << 4); }
 
 struct Group {
   int req, t0, nt, h0;   // request, first token, tokens, first head
@@ -89,13 +87,12 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
   constexpr int KF = DK / 32;          // MFMA k-steps of the score GEMM
   constexpr int WC = LORA / 4;         // value columns per wave
   constexpr int NF = WC / 16;          // 16-column fragments per wave
-  // The 16 B-slot swizzle permutes within 128 B, so it needs rows that
-  // are whole multiples of that; other widths pad the row instead.
-  constexpr bool SWZ = DK % 64 == 0;
-  constexpr int KROW = SWZ ? DK * 2 : DK * 2 + 16;   // bytes
-  auto kaddr = [](int tok, int byte_off) {
-    return tok * KROW + (SWZ ? swz(tok, byte_off) : byte_off);
-  };
+  // Rows of the staged tile are padded by 16 B: with a row stride of
+  // 36 dwords (mod 64 banks) both the token-pair-major stores of the
+  // staging loop and the QK reads (16 rows x 16 B per quarter wave) touch
+  // every bank group equally often, the best a 1 KB access can do.
+  constexpr int KROW = DK * 2 + 16;   // bytes
+  auto kaddr = [](int tok, int byte_off) { return tok * KROW + byte_off; };
 
   const Group grp = find_group(blockIdx.x, qsl, req0, num_reqs, H, tpg, gpt);
   if (grp.nt == 0) return;
@@ -185,42 +182,62 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
   const float sc2 = scale * LOG2E;
   const int* bt = block_table + (long)grp.req * bt_stride;
 
-  for (int sub0 = t_begin; sub0 < t_end; sub0 += SUB) {
-    // ---- stage 32 cached rows. A thread takes one 16 B column chunk of
-    // a PAIR of adjacent tokens: the pair's values go into the
-    // transposed copy as one dword per column, and with token pairs
-    // fastest across lanes and a column stride of VS = 18 dwords a
-    // wave's 64 stores fall on 64 different banks.
-    for (int c = tid; c < (SUB / 2) * (DK / 8); c += THREADS) {
+  // Staging: a thread takes one 16 B column chunk of a PAIR of adjacent
+  // tokens. The pair's values go into the transposed copy as one dword
+  // per column; with token pairs fastest across lanes and a column
+  // stride of VS = 18 dwords a wave's 64 stores fall on 64 different
+  // banks. The global loads of the NEXT subtile are issued before the
+  // current one is computed, so their latency hides behind the MFMAs.
+  constexpr int ITEMS = (SUB / 2) * (DK / 8);
+  constexpr int NIT = (ITEMS + THREADS - 1) / THREADS;
+  s16x8 pre0[NIT], pre1[NIT];
+  const bool bs_pow2 = (block_size & (block_size - 1)) == 0;
+  const int bs_shift = 31 - __builtin_clz(block_size);
+  auto row_of = [&](int t) -> long {
+    const int page = bs_pow2 ? (t >> bs_shift) : t / block_size;
+    const int off = bs_pow2 ? (t & (block_size - 1)) : t % block_size;
+    return ((long)bt[page] * block_size + off) * DK;
+  };
+  auto fetch = [&](int sub0) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = tid + it * THREADS;
       const int tp = c % (SUB / 2);
       const int f8 = c / (SUB / 2);
       const int t_glob = sub0 + 2 * tp;
-      s16x8 v0 = {0, 0, 0, 0, 0, 0, 0, 0};
-      s16x8 v1 = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (t_glob < t_end) {
-        const int blk = bt[t_glob / block_size];
-        v0 = *reinterpret_cast<const s16x8*>(
-            kv + ((long)blk * block_size + t_glob % block_size) * DK +
-            f8 * 8);
-      }
-      if (t_glob + 1 < t_end) {
-        const int blk = bt[(t_glob + 1) / block_size];
-        v1 = *reinterpret_cast<const s16x8*>(
-            kv + ((long)blk * block_size + (t_glob + 1) % block_size) * DK +
-            f8 * 8);
-      }
+      pre0[it] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      pre1[it] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (c < ITEMS && t_glob < t_end)
+        pre0[it] = *reinterpret_cast<const s16x8*>(kv + row_of(t_glob) +
+                                                   f8 * 8);
+      if (c < ITEMS && t_glob + 1 < t_end)
+        pre1[it] = *reinterpret_cast<const s16x8*>(
+            kv + row_of(t_glob + 1) + f8 * 8);
+    }
+  };
+  fetch(t_begin);
+
+  for (int sub0 = t_begin; sub0 < t_end; sub0 += SUB) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = tid + it * THREADS;
+      if (c >= ITEMS) continue;
+      const int tp = c % (SUB / 2);
+      const int f8 = c / (SUB / 2);
       *reinterpret_cast<s16x8*>(reinterpret_cast<char*>(k_lds) +
-                                kaddr(2 * tp, f8 * 16)) = v0;
+                                kaddr(2 * tp, f8 * 16)) = pre0[it];
       *reinterpret_cast<s16x8*>(reinterpret_cast<char*>(k_lds) +
-                                kaddr(2 * tp + 1, f8 * 16)) = v1;
+                                kaddr(2 * tp + 1, f8 * 16)) = pre1[it];
       if (f8 * 8 < LORA) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
           vt_lds[(f8 * 8 + j) * VS + tp] =
-              (uint32_t)(uint16_t)v0[j] | ((uint32_t)(uint16_t)v1[j] << 16);
+              (uint32_t)(uint16_t)pre0[it][j] |
+              ((uint32_t)(uint16_t)pre1[it][j] << 16);
       }
     }
     __syncthreads();
+    if (sub0 + SUB < t_end) fetch(sub0 + SUB);
 
     // ---- QK: S[16 rows x 16 tokens] for (mtile, ntile).
     f32x4 s_frag = {0.f, 0.f, 0.f, 0.f};
