@@ -12,7 +12,8 @@
 //       softmax in fp32 whose running state starts at (m = sink_h,
 //       l = 1): the sink adds exp(sink_h) to the denominator and nothing
 //       to the numerator. Output = sum_j p_j c_j  [T, H, L]. Serves every
-//       dtype; 16-bit batches take the MFMA tile kernel instead
+//       dtype; bf16 batches with 16 B-stepped widths take the MFMA tile
+//       kernel instead
 //       (latent_attention_tiles.hip).
 
 #include <torch/all.h>

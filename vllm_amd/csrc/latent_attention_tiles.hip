@@ -14,6 +14,9 @@
 //   softmax: online, fp32, log2 domain; per-row max/sum shared through
 //            LDS. The running state of partition 0 starts at
 //            (m = sink_h, l = 1) when the layer has a sink.
+// LORA and ROPE are tile widths; the cached row may be narrower (any
+// kv_rank <= LORA and rot_dim <= ROPE in steps of 8), the missing columns
+// are zero in LDS and in the query fragments.
 //   PV : wave w owns value columns [w*LORA/4, (w+1)*LORA/4).
 // The subtile is staged once: [tok][DK] (padded rows, QK reads rows) plus a
 // transposed copy of the first LORA columns [col][token pair] (PV reads
@@ -80,7 +83,8 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
     const float* __restrict__ sink, const float scale, const int H,
     const int block_size, const int req0, const int num_reqs, const int tpg,
     const int gpt,
-    float* __restrict__ tmp_out,   // [T, H, parts, LORA]
+    const int L, const int R,      // actual widths, multiples of 8
+    float* __restrict__ tmp_out,   // [T, H, parts, L]
     float* __restrict__ tmp_lse,   // [T, H, parts, 2]
     const int max_parts) {
   constexpr int DK = LORA + ROPE;
@@ -163,12 +167,13 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
     for (int kf = 0; kf < KF; ++kf) {
       const int f = kf * 32 + l4 * 8;
       s16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (qt >= 0)
-        v = (f < LORA)
-                ? *reinterpret_cast<const s16x8*>(q_abs + qt * qa_st +
-                                                  qh * qa_sh + f)
-                : *reinterpret_cast<const s16x8*>(q_rot + qt * qr_st +
-                                                  qh * qr_sh + (f - LORA));
+      // Columns [L, LORA) and [LORA + R, DK) of the tile are zero.
+      if (qt >= 0 && f < L)
+        v = *reinterpret_cast<const s16x8*>(q_abs + qt * qa_st +
+                                            qh * qa_sh + f);
+      else if (qt >= 0 && f >= LORA && f - LORA < R)
+        v = *reinterpret_cast<const s16x8*>(q_rot + qt * qr_st +
+                                            qh * qr_sh + (f - LORA));
       qfrag[kf] = v;
     }
   }
@@ -196,7 +201,13 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
   auto row_of = [&](int t) -> long {
     const int page = bs_pow2 ? (t >> bs_shift) : t / block_size;
     const int off = bs_pow2 ? (t & (block_size - 1)) : t % block_size;
-    return ((long)bt[page] * block_size + off) * DK;
+    return ((long)bt[page] * block_size + off) * (L + R);
+  };
+  // Tile column chunk f8 -> offset in a cached row, or -1 (zero fill).
+  auto src_col = [&](int f8) -> int {
+    const int col = f8 * 8;
+    if (col < LORA) return col < L ? col : -1;
+    return col - LORA < R ? L + (col - LORA) : -1;
   };
   auto fetch = [&](int sub0) {
 #pragma unroll
@@ -207,12 +218,13 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
       const int t_glob = sub0 + 2 * tp;
       pre0[it] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
       pre1[it] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (c < ITEMS && t_glob < t_end)
+      const int sc = c < ITEMS ? src_col(f8) : -1;
+      if (sc >= 0 && t_glob < t_end)
         pre0[it] = *reinterpret_cast<const s16x8*>(kv + row_of(t_glob) +
-                                                   f8 * 8);
-      if (c < ITEMS && t_glob + 1 < t_end)
+                                                   sc);
+      if (sc >= 0 && t_glob + 1 < t_end)
         pre1[it] = *reinterpret_cast<const s16x8*>(
-            kv + row_of(t_glob + 1) + f8 * 8);
+            kv + row_of(t_glob + 1) + sc);
     }
   };
   fetch(t_begin);
@@ -349,10 +361,11 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
 #pragma unroll
       for (int nf = 0; nf < NF; ++nf) {
         const int col = wave * WC + nf * 16 + l16;
+        if (col >= L) continue;
         if (single)
-          out[oh * LORA + col] = f32_to_bf16(o_acc[mt][nf][r] / l);
+          out[oh * L + col] = f32_to_bf16(o_acc[mt][nf][r] / l);
         else
-          tmp_out[(oh * max_parts + part) * LORA + col] = o_acc[mt][nf][r];
+          tmp_out[(oh * max_parts + part) * L + col] = o_acc[mt][nf][r];
       }
     }
   }
@@ -366,11 +379,10 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
 
 // out[t,h,:] = sum_p w_p tmp[t,h,p,:] / sum_p w_p l_p, w_p = 2^(m_p - max).
 // Decode rows only (token index == request index). Grid (T, H).
-template <int LORA>
 __global__ void latent_tile_reduce_kernel(
     short* __restrict__ out, const float* __restrict__ tmp_out,
     const float* __restrict__ tmp_lse, const int* __restrict__ seq_lens,
-    const int H, const int max_parts) {
+    const int H, const int max_parts, const int LORA) {
   const int t = blockIdx.x;
   const int h = blockIdx.y;
   const int parts = min((seq_lens[t] + PART - 1) / PART, max_parts);
@@ -401,12 +413,12 @@ void latent_check_args(const torch::Tensor& out, const torch::Tensor& q_abs,
                        const torch::Tensor& seq_lens,
                        const c10::optional<torch::Tensor>& sink);
 
+// Any widths in 16 B steps up to the largest tile: the kernel is built
+// for tile widths {64, 128, 256, 512} x {32, 64} and zero-fills the
+// columns a narrower row does not have.
 bool latent_attention_tiles_supported(int64_t kv_rank, int64_t rot_dim) {
-  return (kv_rank == 64 && rot_dim == 32) ||
-         (kv_rank == 128 && rot_dim == 32) ||
-         (kv_rank == 128 && rot_dim == 64) ||
-         (kv_rank == 256 && rot_dim == 64) ||
-         (kv_rank == 512 && rot_dim == 64);
+  return kv_rank >= 8 && kv_rank <= 512 && kv_rank % 8 == 0 &&
+         rot_dim >= 0 && rot_dim <= 64 && rot_dim % 8 == 0;
 }
 
 void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
@@ -427,9 +439,10 @@ void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
               "latent_attention_tiles: unsupported (kv_rank, rot_dim)");
   // 16 B fragment loads.
   TORCH_CHECK(q_abs.stride(0) % 8 == 0 && q_abs.stride(1) % 8 == 0 &&
-              q_rot.stride(0) % 8 == 0 && q_rot.stride(1) % 8 == 0 &&
-              q_rot.storage_offset() % 8 == 0 &&
-              q_abs.storage_offset() % 8 == 0,
+              q_abs.storage_offset() % 8 == 0 &&
+              (R == 0 || (q_rot.stride(0) % 8 == 0 &&
+                          q_rot.stride(1) % 8 == 0 &&
+                          q_rot.storage_offset() % 8 == 0)),
               "latent_attention_tiles: queries must be 16 B aligned");
   const int num_reqs = seq_lens.numel();
   TORCH_CHECK(num_decodes >= 0 && num_decodes <= num_reqs &&
@@ -464,33 +477,37 @@ void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
           block_table.data_ptr<int>(), (int)block_table.stride(0),
           query_start_loc.data_ptr<int>(), seq_lens.data_ptr<int>(),
           sink.has_value() ? sink->data_ptr<float>() : nullptr,
-          (float)scale, H, (int)cache.size(1), req0, nreq, tpg, gpt,
+          (float)scale, H, (int)cache.size(1), req0, nreq, tpg, gpt, L, R,
           nparts > 1 ? tmp_out.data_ptr<float>() : nullptr,
           nparts > 1 ? tmp_lse.data_ptr<float>() : nullptr, nparts);
     };
     if (n_dec > 0) {
       run(0, n_dec, n_dec, parts);
       if (parts > 1)
-        hipLaunchKernelGGL((latent_tile_reduce_kernel<LO>), dim3(n_dec, H),
+        hipLaunchKernelGGL(latent_tile_reduce_kernel, dim3(n_dec, H),
                            dim3(256), 0, stream, (short*)out.data_ptr(),
                            tmp_out.data_ptr<float>(),
                            tmp_lse.data_ptr<float>(),
-                           seq_lens.data_ptr<int>(), H, parts);
+                           seq_lens.data_ptr<int>(), H, parts, L);
     }
     if (num_reqs > n_dec && T > n_dec)
       run(n_dec, num_reqs - n_dec, T - n_dec, 1);
   };
   using std::integral_constant;
-  if (L == 64 && R == 32)
-    launch(integral_constant<int, 64>{}, integral_constant<int, 32>{});
-  else if (L == 128 && R == 32)
-    launch(integral_constant<int, 128>{}, integral_constant<int, 32>{});
-  else if (L == 128 && R == 64)
-    launch(integral_constant<int, 128>{}, integral_constant<int, 64>{});
-  else if (L == 256 && R == 64)
-    launch(integral_constant<int, 256>{}, integral_constant<int, 64>{});
+  auto with_rope = [&](auto lora) {
+    if (R <= 32)
+      launch(lora, integral_constant<int, 32>{});
+    else
+      launch(lora, integral_constant<int, 64>{});
+  };
+  if (L <= 64)
+    with_rope(integral_constant<int, 64>{});
+  else if (L <= 128)
+    with_rope(integral_constant<int, 128>{});
+  else if (L <= 256)
+    with_rope(integral_constant<int, 256>{});
   else
-    launch(integral_constant<int, 512>{}, integral_constant<int, 64>{});
+    with_rope(integral_constant<int, 512>{});
   HIP_CHECK_KERNEL();
 }
 

@@ -494,7 +494,7 @@ def latent_attention(q_abs, q_rot, cache, block_table, query_start_loc,
                     and t.storage_offset() % 8 == 0 and t.stride(2) == 1)
         if not aligned(q_abs):
             q_abs = q_abs.contiguous()
-        if not aligned(q_rot):
+        if R and not aligned(q_rot):
             q_rot = q_rot.contiguous()
         if max_seq_len <= 0:
             max_seq_len = int(seq_lens.max().item())
