@@ -69,14 +69,18 @@ __global__ __launch_bounds__(LB) void latent_rope_cache_write_kernel(
     typename ET<T>::t* __restrict__ cache,
     const int64_t* __restrict__ slot_mapping) {
   __shared__ float scratch[4];
+  // One sine / cosine per pair index, shared by every head and the key.
+  __shared__ float sn_s[LAT_MAX_R / 2], cs_s[LAT_MAX_R / 2];
   const int64_t t = blockIdx.x;
   const float pos = (float)positions[t];
   const int tid = threadIdx.x;
   const int hd = nope + R;
+  for (int i = tid; i < n_pairs; i += LB)
+    sincosf(pos * inv_freq[i], &sn_s[i], &cs_s[i]);
+  __syncthreads();
   for (int idx = tid; idx < H * n_pairs; idx += LB) {
     const int h = idx / n_pairs, i = idx - h * n_pairs;
-    float sn, cs;
-    sincosf(pos * inv_freq[i], &sn, &cs);
+    const float sn = sn_s[i], cs = cs_s[i];
     typename ET<T>::t* p = q + t * q_st + h * hd + nope + 2 * i;
     const float u = ET<T>::ld(p[0]), v = ET<T>::ld(p[1]);
     p[0] = ET<T>::st(u * cs - v * sn);
@@ -97,8 +101,7 @@ __global__ __launch_bounds__(LB) void latent_rope_cache_write_kernel(
   for (int c = tid; c < L; c += LB)
     row[c] = ET<T>::st(ET<T>::ld(d[c]) * inv * norm_w[c]);
   for (int i = tid; i < n_pairs; i += LB) {
-    float sn, cs;
-    sincosf(pos * inv_freq[i], &sn, &cs);
+    const float sn = sn_s[i], cs = cs_s[i];
     const float u = ET<T>::ld(d[L + 2 * i]), v = ET<T>::ld(d[L + 2 * i + 1]);
     row[L + 2 * i] = ET<T>::st(u * cs - v * sn);
     row[L + 2 * i + 1] = ET<T>::st(v * cs + u * sn);
@@ -220,7 +223,8 @@ void latent_rope_cache_write(torch::Tensor q,
   const int T = q.size(0), H = q.size(1);
   const int R = (int)q.size(2) - (int)nope_dim;
   const int n_pairs = inv_freq.numel();
-  TORCH_CHECK(R >= 0 && 2 * n_pairs <= R);
+  TORCH_CHECK(R >= 0 && 2 * n_pairs <= R && R <= LAT_MAX_R,
+              "rotation: dims <= rot_dim <= 256");
   TORCH_CHECK(positions.scalar_type() == torch::kInt64 &&
               positions.is_contiguous() && positions.numel() == T);
   TORCH_CHECK(inv_freq.scalar_type() == torch::kFloat32 &&

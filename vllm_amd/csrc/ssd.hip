@@ -350,6 +350,10 @@ __global__ __launch_bounds__(SB) void ssd_scan_kernel(
   }
 }
 
+// Up to GN_REG gated values per thread stay in registers between the
+// statistics and the output pass; wider groups recompute them.
+constexpr int GN_REG = 4;
+
 template <typename TZ, typename TO>
 __global__ __launch_bounds__(SB) void gated_group_rms_norm_kernel(
     typename ET<TO>::t* __restrict__ out,       // [T, W]
@@ -360,11 +364,26 @@ __global__ __launch_bounds__(SB) void gated_group_rms_norm_kernel(
   __shared__ float scratch[4];
   const int64_t t = blockIdx.x;
   const int c0 = blockIdx.y * Wg;
+  const bool keep = Wg <= SB * GN_REG;
+  float g[GN_REG];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < Wg; c += SB) {
-    const float zz = ET<TZ>::ld(z[t * z_st + c0 + c]);
-    const float v = y[t * W + c0 + c] * (zz / (1.f + expf(-zz)));
-    ss += v * v;
+  if (keep) {
+#pragma unroll
+    for (int k = 0; k < GN_REG; ++k) {
+      const int c = threadIdx.x + k * SB;
+      g[k] = 0.f;
+      if (c < Wg) {
+        const float zz = ET<TZ>::ld(z[t * z_st + c0 + c]);
+        g[k] = y[t * W + c0 + c] * (zz / (1.f + expf(-zz)));
+      }
+      ss += g[k] * g[k];
+    }
+  } else {
+    for (int c = threadIdx.x; c < Wg; c += SB) {
+      const float zz = ET<TZ>::ld(z[t * z_st + c0 + c]);
+      const float v = y[t * W + c0 + c] * (zz / (1.f + expf(-zz)));
+      ss += v * v;
+    }
   }
   ss = wave_reduce_sum(ss);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -372,10 +391,18 @@ __global__ __launch_bounds__(SB) void gated_group_rms_norm_kernel(
   __syncthreads();
   ss = scratch[0] + scratch[1] + scratch[2] + scratch[3];
   const float inv = 1.f / sqrtf(ss / (float)Wg + eps);
-  for (int c = threadIdx.x; c < Wg; c += SB) {
-    const float zz = ET<TZ>::ld(z[t * z_st + c0 + c]);
-    const float v = y[t * W + c0 + c] * (zz / (1.f + expf(-zz)));
-    out[t * W + c0 + c] = ET<TO>::st(v * inv * w[c0 + c]);
+  if (keep) {
+#pragma unroll
+    for (int k = 0; k < GN_REG; ++k) {
+      const int c = threadIdx.x + k * SB;
+      if (c < Wg) out[t * W + c0 + c] = ET<TO>::st(g[k] * inv * w[c0 + c]);
+    }
+  } else {
+    for (int c = threadIdx.x; c < Wg; c += SB) {
+      const float zz = ET<TZ>::ld(z[t * z_st + c0 + c]);
+      const float v = y[t * W + c0 + c] * (zz / (1.f + expf(-zz)));
+      out[t * W + c0 + c] = ET<TO>::st(v * inv * w[c0 + c]);
+    }
   }
 }
 
