@@ -397,6 +397,33 @@ def test_engine_on_gpu(model_g, dtype):
         got, {k: O.forward(cfg, wt, t) for k, t in later.items()}, dtype)
 
 
+def test_engine_rows_narrower_than_the_tile(tmp_path):
+    """Latent rows that run on a wider tile of the MFMA kernel (96 + 16
+    on 128 + 32, 40 + 8 on 64 + 32) with head sizes that leave the
+    rotated query part off a 16 B boundary, through the engine in bf16
+    and fp32, one request in portions beside decode rows."""
+    layers = [
+        O.latent_entry(heads=5, dim=20, rot_dim=16, vdim=12, kv_rank=96,
+                       rot_dims=12, base=5000.0, mlp="dense", ff=48),
+        O.latent_entry(heads=3, dim=24, rot_dim=16, vdim=20, kv_rank=96,
+                       rot_dims=12, base=5000.0, kv_from=0, mlp="moe",
+                       ff=24, experts=4, top=2, shared_ff=16),
+        O.latent_entry(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=40,
+                       mlp=None),
+    ]
+    cfg = O.make_config(layers, vocab=50, width=40, embed_scale=2.0,
+                        softcap=18.0)
+    wt = O.random_weights(cfg, seed=11)
+    path = O.save_model(str(tmp_path / "m"), cfg, wt)
+    reqs = {"a": _tokens(70, 50, 1), "b": _tokens(9, 50, 2),
+            "c": _tokens(150, 50, 3), "d": _tokens(1, 50, 4)}
+    refs = {k: O.forward(cfg, wt, v) for k, v in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        got, _ = run_schedule(path, _mixed_steps(reqs), dtype=dtype,
+                              max_tokens=448, device=DEV)
+        _compare_positions(got, refs, dtype)
+
+
 def test_greedy_generation_on_gpu(model_g):
     from vllm_amd.entrypoints.llm import LLM
     from vllm_amd.sampling_params import SamplingParams
