@@ -72,8 +72,34 @@ DEVINL Group find_group(int g, const int* __restrict__ qsl, int req0,
   return out;
 }
 
-template <int LORA, int ROPE>
-__launch_bounds__(THREADS) __global__ void latent_tile_kernel(
+// Reductions over the 16 lanes of a DPP row (rotations by 8, 4, 2, 1):
+// every lane ends with the result, no LDS crossbar involved.
+template <int CTRL>
+DEVINL float dpp_rot(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+DEVINL float row16_max(float v) {
+  v = fmaxf(v, dpp_rot<0x128>(v));
+  v = fmaxf(v, dpp_rot<0x124>(v));
+  v = fmaxf(v, dpp_rot<0x122>(v));
+  v = fmaxf(v, dpp_rot<0x121>(v));
+  return v;
+}
+DEVINL float row16_add(float v) {
+  v += dpp_rot<0x128>(v);
+  v += dpp_rot<0x124>(v);
+  v += dpp_rot<0x122>(v);
+  v += dpp_rot<0x121>(v);
+  return v;
+}
+
+// MINW = 2 asks for two workgroups per CU (one wave of each per SIMD, at
+// most 256 registers per lane): prompt portions launch thousands of
+// workgroups and gain from the overlap; decode launches about one per CU
+// and is better off with all the registers.
+template <int LORA, int ROPE, int MINW>
+__launch_bounds__(THREADS, MINW) __global__ void latent_tile_kernel(
     short* __restrict__ out,                          // [T, H, LORA]
     const short* __restrict__ q_abs, const long qa_st, const long qa_sh,
     const short* __restrict__ q_rot, const long qr_st, const long qr_sh,
@@ -270,11 +296,7 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       s_val[r] = tok_g < min(t_end, lim[r]) ? s_frag[r] * sc2 : NEG_INF;
-      float v = s_val[r];
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1)
-        v = fmaxf(v, __shfl_xor(v, off, 64));
-      rowmax[r] = v;
+      rowmax[r] = row16_max(s_val[r]);
     }
     if (l16 == 0) {
 #pragma unroll
@@ -299,10 +321,7 @@ __launch_bounds__(THREADS) __global__ void latent_tile_kernel(
           tok_g < min(t_end, lim[r]) ? exp2f(s_val[r] - m_new[r]) : 0.f;
       p_lds[(mtile * 16 + l4 * 4 + r) * SUB + ntile * 16 + l16] =
           f32_to_bf16(p);
-      float v = p;
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-      rowsum[r] = v;
+      rowsum[r] = row16_add(p);
     }
     if (l16 == 0) {
 #pragma unroll
@@ -465,11 +484,12 @@ void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
   auto launch = [&](auto lora, auto rope) {
     constexpr int LO = decltype(lora)::value;
     constexpr int RO = decltype(rope)::value;
-    auto run = [&](int req0, int nreq, int tokens, int nparts) {
+    auto run = [&](int req0, int nreq, int tokens, int nparts, auto minw) {
+      constexpr int MW = decltype(minw)::value;
       const int gx = gpt > 1 ? tokens * gpt
                              : (tokens + tpg - 1) / tpg + nreq;
       hipLaunchKernelGGL(
-          (latent_tile_kernel<LO, RO>), dim3(gx, nparts), dim3(THREADS), 0,
+          (latent_tile_kernel<LO, RO, MW>), dim3(gx, nparts), dim3(THREADS), 0,
           stream, (short*)out.data_ptr(), (const short*)q_abs.data_ptr(),
           (long)q_abs.stride(0), (long)q_abs.stride(1),
           (const short*)q_rot.data_ptr(), (long)q_rot.stride(0),
@@ -482,7 +502,7 @@ void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
           nparts > 1 ? tmp_lse.data_ptr<float>() : nullptr, nparts);
     };
     if (n_dec > 0) {
-      run(0, n_dec, n_dec, parts);
+      run(0, n_dec, n_dec, parts, std::integral_constant<int, 1>{});
       if (parts > 1)
         hipLaunchKernelGGL(latent_tile_reduce_kernel, dim3(n_dec, H),
                            dim3(256), 0, stream, (short*)out.data_ptr(),
@@ -491,7 +511,8 @@ void latent_attention_tiles(torch::Tensor out, torch::Tensor q_abs,
                            seq_lens.data_ptr<int>(), H, parts, L);
     }
     if (num_reqs > n_dec && T > n_dec)
-      run(n_dec, num_reqs - n_dec, T - n_dec, 1);
+      run(n_dec, num_reqs - n_dec, T - n_dec, 1,
+          std::integral_constant<int, 2>{});
   };
   using std::integral_constant;
   auto with_rope = [&](auto lora) {
