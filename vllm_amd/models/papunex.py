@@ -286,8 +286,6 @@ class PapunexForCausalLM(nn.Module):
                 mx.dt_bias.data.copy_(
                     torch.rand(mx.heads, generator=gen) * 2.0 - 3.0)
                 mx.D.data.fill_(1.0)
-            if isinstance(blk.mlp, PapunexMoE) and blk.mlp.shared:
-                blk.mlp.shared_gate.data.mul_(1.0)
 
     def load_hf_weights(self, tensors, config: ModelConfig) -> None:
         """Checkpoint names: embed, final.norm, head, and per layer i
